@@ -1,0 +1,136 @@
+"""`@flex_rnn.jit`: the user-facing decorator.
+
+Same surface and semantics as the reference class
+(/root/reference/flex_rnn/jit.py:7-84): attributes `step, ninputs, nstates,
+noutputs, apply, forward_func, backward_func, fw_meta, bw_meta`, methods
+`naive(*args, dtype=)`, `naive_fp64(*args)`, and `obj(*inputs, *states) ->
+(*outputs, *final_states)`.  Two dispatcher ops are registered per instance,
+`flex_rnn::fw_<id>` and `flex_rnn::bw_<id>`, with fake (meta) implementations and an
+autograd formula, so the object composes with `torch.compile` without graph
+breaks.  Kernels are built lazily on the first real call; a later call with other
+shapes, strides or dtypes fails the metadata check, as in the reference.
+"""
+from __future__ import annotations
+
+import inspect
+import uuid
+
+import torch as th
+
+from .planner import build_twopass, split_list, verify_meta
+
+
+def _tup(x):
+    return x if type(x) == tuple else (x,)
+
+
+class jit:
+    def __init__(self, step, n_step_args=None):
+        self.step = step
+        self.forward_func = self.backward_func = None
+        if n_step_args is None:
+            n_step_args = len(inspect.signature(step).parameters)
+        # arity: run the step once on 1x1 meta tensors (jit.py:13-16)
+        y, s = step(*[th.empty(1, 1, device='meta') for _ in range(n_step_args)])
+        self.noutputs, self.nstates = len(y), len(s)
+        self.ninputs = n_step_args - self.nstates
+        self.apply = self.build_call()
+
+    def __call__(self, *args):
+        return self.apply(*args)
+
+    # ------------------------------------------------------------------ oracle
+    def naive(self, *args, dtype=th.float32):
+        """Pure-PyTorch per-timestep loop with the compiled path's calling convention
+        (jit.py:23-36): inputs are cast to `dtype`, the initial state is not; outputs
+        come back in the step's output dtype under `dtype` inputs, final states in the
+        layout of the initial states."""
+        inputs, state0 = split_list(args, [self.ninputs, self.nstates])
+        state = state0
+        T = max(i.shape[1] for i in inputs)
+        output = None
+        for t in range(T):
+            inputs_t = tuple(i.expand(-1, T, -1, -1, -1)[:, t].to(dtype) for i in inputs)
+            output_t, state = self.step(*inputs_t, *state)
+            output_t, state = _tup(output_t), _tup(state)
+            if output is None:
+                output = tuple(th.empty(o.shape[0], T, o.shape[1], o.shape[2], dtype=o.dtype, device=o.device)
+                               for o in output_t)
+            for dst, src in zip(output, output_t):
+                dst[:, t] = src.squeeze(-1)
+        state = tuple(th.empty_like(x).copy_(y) for x, y in zip(state0, state))
+        return (*output, *state)
+
+    def naive_fp64(self, *args):
+        return self.naive(*args, dtype=th.double)
+
+    # --------------------------------------------------------------- dispatcher
+    def build_call(self):
+        uid = uuid.uuid4().hex
+        nin, nst, nout = self.ninputs, self.nstates, self.noutputs
+        naux = 1        # all saved row-sums travel in one packed tensor (jit.py:43)
+
+        def metas(meta, device):
+            return tuple(th.empty_strided(shape, stride, dtype=dtype, device=device) for shape, stride, dtype in meta)
+
+        fw_schema = '(' + ', '.join(f'Tensor x{i}' for i in range(nin + nst)) + ') -> (' \
+            + ', '.join(['Tensor'] * (nout + 2 * nst + naux)) + ')'
+
+        @th.library.custom_op('flex_rnn::fw_' + uid, mutates_args=(), schema=fw_schema)
+        def apply(*args):
+            inputs, state = split_list(args, [nin, nst])
+            if self.forward_func is None:
+                self.forward_func, self.backward_func, self.fw_meta, self.bw_meta = \
+                    build_twopass(self.step, inputs, state)
+            r = self.forward_func(inputs, state)
+            verify_meta(r, metas(self.fw_meta, 'meta'))
+            return r
+
+        @apply.register_fake
+        def _(*args):
+            inputs, state = split_list(args, [nin, nst])
+            if not hasattr(self, 'fw_meta'):
+                self.fw_meta, self.bw_meta = build_twopass(self.step, inputs, state, dryrun=True)
+            return metas(self.fw_meta, args[0].device)
+
+        bw_schema = '(' + ', '.join(f'Tensor x{i}' for i in range(nout + 2 * nst + nin + naux)) + ') -> (' \
+            + ', '.join(['Tensor'] * (nin + nst)) + ')'
+
+        @th.library.custom_op('flex_rnn::bw_' + uid, mutates_args=(), schema=bw_schema)
+        def backward_inner(*args):
+            doutput, dstateT, inputs, state_store, aux = split_list(args, [nout, nst, nin, nst, naux])
+            dinputs, dstate0 = self.backward_func(doutput, dstateT, inputs, state_store, aux)
+            verify_meta(dinputs + dstate0, metas(self.bw_meta, 'meta'))
+            return (*dinputs, *dstate0)
+
+        @backward_inner.register_fake
+        def _(*args):
+            return metas(self.bw_meta, args[0].device)
+
+        def setup_context(ctx, inputs, output):
+            ctx.set_materialize_grads(False)
+            ctx.save_for_backward(*inputs[:nin], *output[nout + nst:])
+            ctx.output_meta = tuple(o.to('meta') for o in output[:nout + nst])
+
+        def backward(ctx, *grads):
+            grads = list(grads)
+            for i, meta in enumerate(ctx.output_meta):
+                if grads[i] is None:
+                    grads[i] = th.zeros_like(meta, device=ctx.saved_tensors[0].device)
+            return backward_inner(*grads[:nout + nst], *ctx.saved_tensors)
+
+        apply.register_autograd(backward, setup_context=setup_context)
+        self._fw_op, self._bw_op = apply, backward_inner
+        return lambda *args: apply(*args)[:nout + nst]
+
+
+def simplified_naive(step, *args):
+    """Single-state, single-output loop shown in the reference's README (jit.py:86-94)."""
+    inputs, state = args[:-1], args[-1]
+    T = max(i.shape[1] for i in inputs)
+    ys = []
+    for t in range(T):
+        xs = [i.expand(-1, T, -1, -1, -1)[:, t].float() for i in inputs]
+        y, state = step(*xs, state)
+        ys.append(y)
+    return th.stack(ys, dim=1).squeeze(-1), state

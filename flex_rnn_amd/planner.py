@@ -1,0 +1,258 @@
+"""Planner: validates the call, classifies operands, traces + partitions the step,
+chooses tile sizes and hidden-buffer layouts, and (unless `dryrun`) builds the
+HIP kernels and returns the `forward` / `backward` closures.
+
+Interface and behaviour follow /root/reference/flex_rnn/twopass.py:
+  * `split_list`, `get_meta`, `verify_meta`                     (twopass.py:8-15, 33-42)
+  * `build_twopass(step, inputs, state, dryrun=False)`           (twopass.py:44-366)
+      -> (forward, backward, forward_meta, backward_meta)  or the two metas when dryrun
+  * `forward(inputs, state) -> (*y, *stateT, *state_store, aux)` (twopass.py:224-237)
+  * `backward(doutput, dstateT, inputs, state_store, aux)
+        -> (tuple(dinputs), tuple(dstate0))`                     (twopass.py:343-363)
+The kernels, their tiling and the layout of the hidden buffers (`state_store`,
+`aux`) are this backend's own.
+"""
+from __future__ import annotations
+
+import hashlib
+from dataclasses import dataclass, field
+from typing import Callable, Dict, List, Optional, Sequence, Tuple
+
+import torch as th
+
+from . import tracer
+from .partition import Partition, partition
+
+SUPPORTED_DTYPES = (th.float32, th.bfloat16, th.float16, th.float64)
+
+
+def split_list(args, lens):
+    """Cut `args` into consecutive pieces of the given lengths (twopass.py:8-15)."""
+    out, off = [], 0
+    for n in lens:
+        out.append(args[off:off + n])
+        off += n
+    assert off == len(args), f'expected {off} arguments, got {len(args)}'
+    return out
+
+
+def get_meta(tensors):
+    return tuple((t.shape, t.stride(), t.dtype) for t in tensors)
+
+
+def _eff_stride(shape, stride):
+    return [s if n > 1 else 0 for s, n in zip(stride, shape)]
+
+
+def verify_meta(a, b, msg=''):
+    """Shapes, dtypes and strides (ignoring size-1 dims) must agree (twopass.py:36-42)."""
+    for i, ((ash, ast, adt), (bsh, bst, bdt)) in enumerate(zip(get_meta(a), get_meta(b))):
+        assert ash == bsh, msg + f'#{i+1}: a_shape={ash} != b_shape={bsh}'
+        a_stride, b_stride = _eff_stride(ash, ast), _eff_stride(bsh, bst)
+        assert a_stride == b_stride, msg + f'#{i+1}: {a_stride=} != {b_stride=}'
+        assert adt == bdt, msg + f'#{i+1}: a_dtype={adt} != b_dtype={bdt}'
+
+
+def _pow2_floor(n: int) -> int:
+    return 1 << (max(int(n), 1).bit_length() - 1)
+
+
+def _is_pow2(n: int) -> bool:
+    return n >= 1 and (n & (n - 1)) == 0
+
+
+@dataclass
+class TileConfig:
+    """Launch geometry of the three kernels.
+
+    Row kernels (fw, bw1): a wave holds G = 64/L row groups; each group of L lanes holds
+    R consecutive state rows, each lane C = N/L columns of them.  W waves per workgroup, so a
+    workgroup owns MT = W*G*R rows of one (batch, head).  Inputs are staged through LDS TS
+    timesteps at a time; the state is checkpointed every DT steps.
+    Gradient kernel (bw2): one lane per state column, DT timesteps per instance, a serial
+    loop over the M rows."""
+    L: int
+    C: int
+    R: int
+    W: int
+    DT: int
+    TS: int
+    R1: int = 0          # rows per lane / waves in bw1 (0 = same as fw)
+    W1: int = 0
+
+    @property
+    def G(self): return 64 // self.L
+    @property
+    def MT(self): return self.W * self.G * self.R
+
+
+@dataclass
+class Plan:
+    B: int
+    T: int
+    H: int
+    M: int
+    N: int
+    part: Partition
+    in_cls: List[str]
+    in_dtypes: List[th.dtype]
+    in_bcast: List[Tuple[bool, bool, bool]]     # input broadcast over (B, T, H)
+    st_dtypes: List[th.dtype]
+    out_dtypes: List[th.dtype]
+    tile: TileConfig
+    nchunks: int
+
+    @property
+    def atomic(self) -> List[int]:
+        return [i for i, b in enumerate(self.in_bcast) if any(b)]
+
+
+def classify(inputs, state):
+    """Shape validation and operand classes (twopass.py:45-72)."""
+    B, T, H = [max(i.shape[j] for i in inputs) for j in range(3)]
+    M = max(i.shape[-2] for i in tuple(inputs) + tuple(state))
+    N = max(i.shape[-1] for i in tuple(inputs) + tuple(state))
+    dims = [B, T, H, M, N]
+    for i, x in enumerate(inputs):
+        assert x.ndim == 5, f'invalid shape {list(x.shape)} of argument #{i+1}'
+        for j in range(5):
+            assert x.shape[j] in [1, dims[j]], \
+                f'shape {list(x.shape)} of argument #{i+1} is incompatible with {dims}'
+        assert 1 in x.shape[-2:] or x.shape[1] == 1, \
+            f'shape {list(x.shape)} of argument #{i+1} is both a matrix for each head, and depends on time. This is not supported'
+        assert x.dtype in SUPPORTED_DTYPES, f'unsupported dtype {x.dtype} of argument #{i+1}'
+    for i, x in enumerate(state):
+        assert list(x.shape) == [B, H, M, N], \
+            f'shape {list(x.shape)} of argument #{i+1+len(inputs)} != {[B, H, M, N]}'
+        assert x.dtype in SUPPORTED_DTYPES, f'unsupported dtype {x.dtype} of argument #{i+1+len(inputs)}'
+    cls = []
+    for x in inputs:
+        mn = list(x.shape[-2:])
+        if mn == [1, 1]:
+            cls.append('scalar')
+        elif mn == [M, 1]:
+            cls.append('col')
+        elif mn == [1, N]:
+            cls.append('row')
+        else:
+            assert mn == [M, N]
+            cls.append('mat')
+    bcast = [tuple(x.shape[j] == 1 and dims[j] != 1 for j in range(3)) for x in inputs]
+    return dims, cls, bcast
+
+
+def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256) -> TileConfig:
+    """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
+    assert _is_pow2(N), f'state width N={N} must be a power of two'
+    assert _is_pow2(M), f'state height M={M} must be a power of two'
+    # columns per lane: up to 8 so that a row of up to 128 columns fits one 16-lane DPP row
+    C = min(N, 8)
+    L = N // C
+    while L > 64:
+        C *= 2
+        L = N // C
+    G = 64 // L
+    nst = part.nstates + len(part.mat_idx)
+    # rows per lane: bounded by the register budget (state + new state + a few temporaries)
+    R = max(1, min(64 // max(C * nst, 1), 8))
+    R = _pow2_floor(R)
+    # do not give a wave more rows than exist
+    while R > 1 and G * R > M:
+        R //= 2
+    rows_per_wave = G * R
+    if rows_per_wave > M:
+        # fewer rows than row groups: leave groups idle (handled by row masking)
+        W = 1
+    else:
+        W = max(1, min(4, M // rows_per_wave))
+    # enough workgroups to fill the chip: shrink R while the grid is small
+    def nwg(R_, W_):
+        return B * H * max(1, M // (W_ * G * R_))
+    while R > 1 and nwg(R, W) * W < 4 * n_cu:
+        R //= 2
+        W = max(1, min(4, M // (G * R)))
+    per_step_regs = 0
+    for i, c in enumerate(part_input_classes(part)):
+        per_step_regs += 1
+    DT = 16
+    if part.dstep_needs_state:
+        DT = 8
+    while DT > 1 and T % DT != 0:
+        DT //= 2
+    TS = min(DT, 8)
+    if part.dstep_needs_state:
+        TS = DT
+    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS)
+
+
+def part_input_classes(part: Partition) -> List[str]:
+    cls = [None] * part.ninputs
+    for name, idx in (('col', part.col_idx), ('row', part.row_idx), ('scalar', part.scalar_idx), ('mat', part.mat_idx)):
+        for i in idx:
+            cls[i] = name
+    return cls
+
+
+def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) -> Tuple[Plan, tuple, tuple]:
+    (B, T, H, M, N), cls, bcast = classify(inputs, state)
+
+    inputs_t = [i[:, 0] for i in inputs]
+    res = step(*[i.to('meta') for i in [*inputs_t, *state]])
+    output_t, nstate = [r if isinstance(r, tuple) else (r,) for r in res]
+    ninputs, noutputs, nstates = len(inputs_t), len(output_t), len(nstate)
+    assert len(nstate) == len(state), 'step must return as many states as it takes'
+    assert all(a.shape == b.shape for a, b in zip(nstate, state)), 'new state shape differs from the state shape'
+    assert all(list(i.shape) == [B, H, M, 1] for i in output_t), [i.shape for i in output_t]
+    assert all(i.dtype in SUPPORTED_DTYPES for i in output_t)
+
+    metas = tuple(th.empty(j.shape[-2:], dtype=j.dtype, device='meta') for j in tuple(inputs_t) + tuple(state))
+    joint, nfw = tracer.trace_step(step, metas)
+    assert nfw == noutputs + nstates
+    part = partition(joint, ninputs, nstates, noutputs, cls)
+
+    if tile is None:
+        tile = choose_tiles(B, T, H, M, N, part)
+    assert T % tile.DT == 0 and tile.DT % tile.TS == 0
+    nchunks = T // tile.DT
+    plan = Plan(B, T, H, M, N, part, cls, [i.dtype for i in inputs], bcast,
+                [s.dtype for s in state], [o.dtype for o in output_t], tile, nchunks)
+
+    dev = 'meta'
+    output_out = tuple(th.empty(B, T, H, M, dtype=o.dtype, device=dev) for o in output_t)
+    dstate = tuple(th.empty_like(s, device=dev) for s in state)
+    state_store = tuple(th.empty(B, H, nchunks, M, N, dtype=th.float32, device=dev) for _ in state)
+    aux_out = (th.empty(len(part.aux), B, H, T, M, dtype=th.float32, device=dev),)
+    dinputs_out = tuple(th.empty_like(i, device=dev) for i in inputs)
+    forward_meta = get_meta([*output_out, *dstate, *state_store, *aux_out])
+    backward_meta = get_meta([*dinputs_out, *dstate])
+    return plan, forward_meta, backward_meta
+
+
+def build_twopass(step: Callable, inputs, state, dryrun: bool = False, tile: Optional[TileConfig] = None):
+    inputs, state = tuple(inputs), tuple(state)
+    plan, forward_meta, backward_meta = make_plan(step, inputs, state, tile)
+    if dryrun:
+        return forward_meta, backward_meta
+
+    from .launch import CompiledPlan
+    compiled = CompiledPlan(plan)
+
+    in_meta = tuple(th.empty_strided(i.shape, i.stride(), dtype=i.dtype, device='meta') for i in inputs)
+    st_meta = tuple(th.empty_strided(s.shape, s.stride(), dtype=s.dtype, device='meta') for s in state)
+    fw_out_meta = tuple(th.empty_strided(sh, st, dtype=dt, device='meta') for sh, st, dt in forward_meta)
+    nout, nst = plan.part.noutputs, plan.part.nstates
+
+    def forward(inputs_, state0):
+        verify_meta(inputs_, in_meta, 'input Tensor metadata doesn\'t match compilation\n')
+        verify_meta(state0, st_meta, 'initial state Tensor metadata doesn\'t match compilation\n')
+        return compiled.forward(tuple(inputs_), tuple(state0))
+
+    def backward(doutput, dstateT_, inputs_, state_store_, aux_):
+        doutput, dstateT_ = [tuple(i.contiguous() for i in j) for j in (doutput, dstateT_)]
+        verify_meta(inputs_, in_meta)
+        verify_meta(doutput, fw_out_meta[:nout])
+        verify_meta(state_store_, fw_out_meta[nout + nst:nout + 2 * nst])
+        verify_meta(aux_, fw_out_meta[nout + 2 * nst:])
+        return compiled.backward(doutput, dstateT_, tuple(inputs_), tuple(state_store_), aux_[0])
+
+    return forward, backward, forward_meta, backward_meta
