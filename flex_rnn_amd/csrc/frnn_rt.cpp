@@ -1,0 +1,300 @@
+// frnn_rt: C-ABI runtime for generated gfx950 kernels (see include/frnn_rt.h).
+//
+// Host-only C++; the HIP runtime is resolved at run time from the process image
+// (dlsym(RTLD_DEFAULT)) so that the copy PyTorch already loaded is the one used, and is
+// dlopen'ed by soname only when the process has none.
+#include "frnn_rt.h"
+
+#include <dlfcn.h>
+#include <errno.h>
+#include <fcntl.h>
+#include <spawn.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <sys/file.h>
+#include <sys/stat.h>
+#include <sys/wait.h>
+#include <unistd.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+extern char** environ;
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[4096];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+// ---------------------------------------------------------------- HIP entry points
+typedef int hipError_t;
+struct HipApi {
+  hipError_t (*ModuleLoad)(void**, const char*) = nullptr;
+  hipError_t (*ModuleUnload)(void*) = nullptr;
+  hipError_t (*ModuleGetFunction)(void**, void*, const char*) = nullptr;
+  hipError_t (*ModuleLaunchKernel)(void*, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned,
+                                   unsigned, void*, void**, void**) = nullptr;
+  const char* (*GetErrorString)(hipError_t) = nullptr;
+  hipError_t (*GetDevice)(int*) = nullptr;
+  hipError_t (*DeviceGetAttribute)(int*, int, int) = nullptr;
+  hipError_t (*GetLastError)() = nullptr;
+  bool ok = false;
+  std::string why;
+};
+
+HipApi& hip() {
+  static HipApi api;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    void* h = RTLD_DEFAULT;
+    if (!dlsym(RTLD_DEFAULT, "hipModuleLoad")) {
+      h = dlopen("libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+      if (!h) h = dlopen("libamdhip64.so.7", RTLD_NOW | RTLD_GLOBAL);
+      if (!h) h = dlopen("/opt/rocm/lib/libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
+      if (!h) {
+        api.why = "no HIP runtime in the process and libamdhip64.so could not be loaded";
+        return;
+      }
+    }
+#define FRNN_SYM(field, name)                                              \
+  *(void**)(&api.field) = dlsym(h, name);                                  \
+  if (!api.field) { api.why = std::string("missing HIP symbol ") + name; return; }
+    FRNN_SYM(ModuleLoad, "hipModuleLoad")
+    FRNN_SYM(ModuleUnload, "hipModuleUnload")
+    FRNN_SYM(ModuleGetFunction, "hipModuleGetFunction")
+    FRNN_SYM(ModuleLaunchKernel, "hipModuleLaunchKernel")
+    FRNN_SYM(GetErrorString, "hipGetErrorString")
+    FRNN_SYM(GetDevice, "hipGetDevice")
+    FRNN_SYM(DeviceGetAttribute, "hipDeviceGetAttribute")
+    FRNN_SYM(GetLastError, "hipGetLastError")
+#undef FRNN_SYM
+    api.ok = true;
+  });
+  return api;
+}
+
+int hip_fail(const char* what, hipError_t e) {
+  const char* s = hip().GetErrorString ? hip().GetErrorString(e) : "?";
+  return fail(FRNN_ERR_HIP, "%s failed: %s (%d)", what, s, (int)e);
+}
+
+// ---------------------------------------------------------------- small file helpers
+bool file_exists(const std::string& p) {
+  struct stat st;
+  return stat(p.c_str(), &st) == 0 && S_ISREG(st.st_mode) && st.st_size > 0;
+}
+
+int mkdirs(const std::string& dir) {
+  std::string cur;
+  for (size_t i = 0; i <= dir.size(); i++) {
+    if (i == dir.size() || dir[i] == '/') {
+      if (!cur.empty() && mkdir(cur.c_str(), 0777) != 0 && errno != EEXIST) return -1;
+    }
+    if (i < dir.size()) cur.push_back(dir[i]);
+  }
+  return 0;
+}
+
+int write_file(const std::string& path, const char* data, size_t len) {
+  FILE* f = fopen(path.c_str(), "wb");
+  if (!f) return -1;
+  size_t w = fwrite(data, 1, len, f);
+  int rc = fclose(f);
+  return (w == len && rc == 0) ? 0 : -1;
+}
+
+std::string read_tail(const std::string& path, size_t maxb) {
+  FILE* f = fopen(path.c_str(), "rb");
+  if (!f) return "";
+  fseek(f, 0, SEEK_END);
+  long n = ftell(f);
+  long off = n > (long)maxb ? n - (long)maxb : 0;
+  fseek(f, off, SEEK_SET);
+  std::string s((size_t)(n - off), '\0');
+  size_t r = fread(&s[0], 1, s.size(), f);
+  s.resize(r);
+  fclose(f);
+  return s;
+}
+
+std::string find_hipcc() {
+  if (const char* e = getenv("FRNN_HIPCC")) return e;
+  if (const char* r = getenv("ROCM_PATH")) {
+    std::string p = std::string(r) + "/bin/hipcc";
+    if (access(p.c_str(), X_OK) == 0) return p;
+  }
+  if (access("/opt/rocm/bin/hipcc", X_OK) == 0) return "/opt/rocm/bin/hipcc";
+  return "hipcc";
+}
+
+std::vector<std::string> split_ws(const char* s) {
+  std::vector<std::string> out;
+  if (!s) return out;
+  std::string cur;
+  for (const char* p = s;; p++) {
+    if (*p == 0 || *p == ' ' || *p == '\t' || *p == '\n') {
+      if (!cur.empty()) out.push_back(cur);
+      cur.clear();
+      if (*p == 0) break;
+    } else {
+      cur.push_back(*p);
+    }
+  }
+  return out;
+}
+
+}  // namespace
+
+struct frnn_module_s {
+  void* mod;
+};
+
+extern "C" {
+
+int frnn_version(void) { return 100; }
+
+const char* frnn_last_error(void) { return g_err.c_str(); }
+
+int frnn_compile(const char* src, size_t len, const char* arch, const char* opts,
+                 const char* cache_dir, const char* key, char* out_path, size_t cap) {
+  if (!src || !arch || !cache_dir || !key || !out_path || cap == 0)
+    return fail(FRNN_ERR_ARG, "frnn_compile: null argument");
+  for (const char* p = key; *p; p++)
+    if (!((*p >= 'a' && *p <= 'z') || (*p >= 'A' && *p <= 'Z') || (*p >= '0' && *p <= '9') || *p == '_' || *p == '-'))
+      return fail(FRNN_ERR_ARG, "frnn_compile: key may only hold [A-Za-z0-9_-]");
+  std::string dir(cache_dir);
+  if (mkdirs(dir) != 0) return fail(FRNN_ERR_IO, "cannot create cache directory %s: %s", cache_dir, strerror(errno));
+  std::string base = dir + "/" + key;
+  std::string hsaco = base + ".hsaco";
+  if (hsaco.size() + 1 > cap) return fail(FRNN_ERR_ARG, "frnn_compile: out_path too small");
+  strcpy(out_path, hsaco.c_str());
+  if (file_exists(hsaco)) return FRNN_OK;
+
+  // serialise concurrent builders of the same key
+  std::string lockp = base + ".lock";
+  int lockfd = open(lockp.c_str(), O_CREAT | O_RDWR, 0666);
+  if (lockfd < 0) return fail(FRNN_ERR_IO, "cannot open lock file %s: %s", lockp.c_str(), strerror(errno));
+  if (flock(lockfd, LOCK_EX) != 0) {
+    close(lockfd);
+    return fail(FRNN_ERR_IO, "cannot lock %s: %s", lockp.c_str(), strerror(errno));
+  }
+  struct Unlock {
+    int fd;
+    ~Unlock() { flock(fd, LOCK_UN); close(fd); }
+  } unlock{lockfd};
+  if (file_exists(hsaco)) return FRNN_OK;   // someone else built it while we waited
+
+  std::string srcp = base + ".hip";
+  if (write_file(srcp, src, len) != 0) return fail(FRNN_ERR_IO, "cannot write %s: %s", srcp.c_str(), strerror(errno));
+  char tmpn[64];
+  snprintf(tmpn, sizeof tmpn, ".tmp%d", (int)getpid());
+  std::string tmpo = hsaco + tmpn;
+  std::string logp = base + ".log";
+
+  std::vector<std::string> av = {find_hipcc(), "--genco", std::string("--offload-arch=") + arch, "-O3", "-std=c++17",
+                                 // packed fp32 VALU ops are kept off on this hardware pool
+                                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  for (auto& o : split_ws(opts)) av.push_back(o);
+  av.push_back("-o");
+  av.push_back(tmpo);
+  av.push_back(srcp);
+  std::vector<char*> argv;
+  for (auto& s : av) argv.push_back(const_cast<char*>(s.c_str()));
+  argv.push_back(nullptr);
+
+  posix_spawn_file_actions_t fa;
+  posix_spawn_file_actions_init(&fa);
+  posix_spawn_file_actions_addopen(&fa, 1, logp.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0666);
+  posix_spawn_file_actions_adddup2(&fa, 1, 2);
+  pid_t pid;
+  int rc = posix_spawnp(&pid, argv[0], &fa, nullptr, argv.data(), environ);
+  posix_spawn_file_actions_destroy(&fa);
+  if (rc != 0) return fail(FRNN_ERR_COMPILE, "cannot start %s: %s", argv[0], strerror(rc));
+  int status = 0;
+  while (waitpid(pid, &status, 0) < 0) {
+    if (errno != EINTR) return fail(FRNN_ERR_COMPILE, "waitpid failed: %s", strerror(errno));
+  }
+  if (!WIFEXITED(status) || WEXITSTATUS(status) != 0 || !file_exists(tmpo)) {
+    std::string log = read_tail(logp, 3000);
+    unlink(tmpo.c_str());
+    return fail(FRNN_ERR_COMPILE, "hipcc failed (status %d) for %s:\n%s", status, srcp.c_str(), log.c_str());
+  }
+  if (rename(tmpo.c_str(), hsaco.c_str()) != 0) {
+    unlink(tmpo.c_str());
+    return fail(FRNN_ERR_IO, "cannot rename %s: %s", tmpo.c_str(), strerror(errno));
+  }
+  return FRNN_OK;
+}
+
+int frnn_module_load(const char* path, frnn_module_t* out) {
+  if (!path || !out) return fail(FRNN_ERR_ARG, "frnn_module_load: null argument");
+  HipApi& h = hip();
+  if (!h.ok) return fail(FRNN_ERR_NO_HIP, "%s", h.why.c_str());
+  void* mod = nullptr;
+  hipError_t e = h.ModuleLoad(&mod, path);
+  if (e != 0) return hip_fail("hipModuleLoad", e);
+  *out = new frnn_module_s{mod};
+  return FRNN_OK;
+}
+
+int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out) {
+  if (!m || !name || !out) return fail(FRNN_ERR_ARG, "frnn_get_kernel: null argument");
+  HipApi& h = hip();
+  if (!h.ok) return fail(FRNN_ERR_NO_HIP, "%s", h.why.c_str());
+  void* fn = nullptr;
+  hipError_t e = h.ModuleGetFunction(&fn, m->mod, name);
+  if (e != 0) return hip_fail("hipModuleGetFunction", e);
+  *out = fn;
+  return FRNN_OK;
+}
+
+int frnn_launch(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3],
+                uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes) {
+  if (!k || !grid || !block || (!args && arg_bytes)) return fail(FRNN_ERR_ARG, "frnn_launch: null argument");
+  for (int i = 0; i < 3; i++)
+    if (grid[i] == 0 || block[i] == 0) return fail(FRNN_ERR_ARG, "frnn_launch: empty grid or block");
+  if ((uint64_t)block[0] * block[1] * block[2] > 1024) return fail(FRNN_ERR_ARG, "frnn_launch: block larger than 1024 threads");
+  if (grid[1] > 65535 || grid[2] > 65535) return fail(FRNN_ERR_ARG, "frnn_launch: grid y/z larger than 65535");
+  HipApi& h = hip();
+  if (!h.ok) return fail(FRNN_ERR_NO_HIP, "%s", h.why.c_str());
+  size_t sz = arg_bytes;
+  void* extra[] = {(void*)0x01 /*BUFFER_POINTER*/, const_cast<void*>(args), (void*)0x02 /*BUFFER_SIZE*/, &sz,
+                   (void*)0x03 /*END*/};
+  hipError_t e = h.ModuleLaunchKernel(k, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, stream,
+                                      nullptr, extra);
+  if (e != 0) return hip_fail("hipModuleLaunchKernel", e);
+  return FRNN_OK;
+}
+
+int frnn_module_free(frnn_module_t m) {
+  if (!m) return FRNN_OK;
+  HipApi& h = hip();
+  hipError_t e = 0;
+  if (h.ok && m->mod) e = h.ModuleUnload(m->mod);
+  delete m;
+  if (e != 0) return hip_fail("hipModuleUnload", e);
+  return FRNN_OK;
+}
+
+int frnn_device_cus(void) {
+  HipApi& h = hip();
+  if (!h.ok) return -1;
+  int dev = 0, cus = 0;
+  if (h.GetDevice(&dev) != 0) return -1;
+  if (h.DeviceGetAttribute(&cus, 63 /*hipDeviceAttributeMultiprocessorCount*/, dev) != 0) return -1;
+  return cus;
+}
+
+}  // extern "C"

@@ -1,0 +1,814 @@
+"""HIP (gfx950, wave64) code emitter for the three kernels of a plan.
+
+Replaces the reference's CUDA text emitter (/root/reference/flex_rnn/to_cuda.py:7-124
+`to_cuda`, 127-223 `parse_cuda`) and its three kernel templates
+(/root/reference/flex_rnn/twopass.py:202-220 `fw`, 245-273 `bw1`, 285-339 `bw2`).
+Nothing of their thread mapping is kept:
+
+  * Row kernels (`fw`, `bw1`): a 64-lane wave is split into G = 64/L row groups of L
+    lanes; a group holds R consecutive state rows in fp32 registers, C = N/L columns per
+    lane.  `sum(-1)` is an in-lane chain over C followed by a DPP all-reduce inside the
+    group (no LDS, no barrier).  Per-timestep operands are staged through LDS as fp32,
+    TS timesteps at a time, by all threads of the workgroup (any stride / dtype is handled
+    there); results go back the same way.
+  * Gradient kernel (`bw2`): one lane per state column and DT timesteps per instance; a
+    serial loop over the M rows recomputes the DT states of one element from its
+    checkpoint (elementwise thanks to the saved row sums), runs the per-element backward,
+    and accumulates the sums over rows in registers.  An epilogue maps them to row /
+    scalar input gradients (column sums = wave all-reduce).
+
+Shapes B, T, H, M and all strides are runtime kernel arguments; N, dtypes, operand
+classes, broadcast pattern and tile sizes are baked into the source (and hence into the
+cache key, which is a hash of the source).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Dict, List, Sequence, Tuple
+
+import torch as th
+
+from .ir import Graph, Node
+
+DT_CODE = {th.float32: 0, th.bfloat16: 1, th.float16: 2, th.float64: 3}
+
+PRELUDE = r'''
+#include <hip/hip_runtime.h>
+typedef long long i64;
+typedef unsigned short u16_t;
+struct TArg { void* p; i64 s[5]; };
+
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xf, 0xf, true));
+}
+// Sum over the L (power of two) consecutive lanes of a group; every lane gets the total.
+// quad_perm / row_half_mirror / row_mirror stay inside a 16-lane DPP row; wider groups
+// cross rows with a lane permute.
+template <int L> __device__ __forceinline__ float grp_allreduce(float x) {
+  if constexpr (L >= 2) x += dpp_mov<0xB1>(x);    // quad_perm [1,0,3,2]
+  if constexpr (L >= 4) x += dpp_mov<0x4E>(x);    // quad_perm [2,3,0,1]
+  if constexpr (L >= 8) x += dpp_mov<0x141>(x);   // row_half_mirror
+  if constexpr (L >= 16) x += dpp_mov<0x140>(x);  // row_mirror
+  if constexpr (L >= 32) x += __shfl_xor(x, 16, 64);
+  if constexpr (L >= 64) x += __shfl_xor(x, 32, 64);
+  return x;
+}
+
+template <int DT> __device__ __forceinline__ float ldf(const void* p, i64 i);
+template <> __device__ __forceinline__ float ldf<0>(const void* p, i64 i) { return ((const float*)p)[i]; }
+template <> __device__ __forceinline__ float ldf<1>(const void* p, i64 i) {
+  return __builtin_bit_cast(float, (unsigned)((const u16_t*)p)[i] << 16);
+}
+template <> __device__ __forceinline__ float ldf<2>(const void* p, i64 i) { return (float)((const _Float16*)p)[i]; }
+template <> __device__ __forceinline__ float ldf<3>(const void* p, i64 i) { return (float)((const double*)p)[i]; }
+
+template <int DT> __device__ __forceinline__ void stf(void* p, i64 i, float v);
+template <> __device__ __forceinline__ void stf<0>(void* p, i64 i, float v) { ((float*)p)[i] = v; }
+template <> __device__ __forceinline__ void stf<1>(void* p, i64 i, float v) {
+  ((u16_t*)p)[i] = __builtin_bit_cast(u16_t, (__bf16)v);
+}
+template <> __device__ __forceinline__ void stf<2>(void* p, i64 i, float v) { ((_Float16*)p)[i] = (_Float16)v; }
+template <> __device__ __forceinline__ void stf<3>(void* p, i64 i, float v) { ((double*)p)[i] = (double)v; }
+
+__device__ __forceinline__ void atomic_addf(void* p, i64 i, float v) {
+  __hip_atomic_fetch_add(((float*)p) + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float f_sigmoid(float x) { return 1.0f / (1.0f + __expf(-x)); }
+__device__ __forceinline__ float f_tanh(float x) { return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f); }
+__device__ __forceinline__ float f_sign(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f); }
+'''
+
+
+def _lit(v) -> str:
+    v = float(v)
+    if math.isinf(v):
+        return '__builtin_inff()' if v > 0 else '(-__builtin_inff())'
+    if math.isnan(v):
+        return '__builtin_nanf("")'
+    s = repr(v)
+    if 'e' not in s and '.' not in s:
+        s += '.0'
+    return s + 'f'
+
+
+_UNARY_EXPR = {
+    'exp': '__expf({0})', 'neg': '(-{0})', 'reciprocal': '(1.0f / {0})', 'log': '__logf({0})',
+    'sqrt': 'sqrtf({0})', 'rsqrt': 'rsqrtf({0})', 'sigmoid': 'f_sigmoid({0})', 'tanh': 'f_tanh({0})',
+    'abs': '__builtin_fabsf({0})', 'relu': 'fmaxf({0}, 0.0f)', 'sign': 'f_sign({0})',
+    'log1p': 'log1pf({0})', 'expm1': 'expm1f({0})', 'copy': '({0})',
+}
+_BINARY_EXPR = {
+    'mul': '({0} * {1})', 'add': '({0} + {1})', 'sub': '({0} - {1})', 'div': '({0} / {1})',
+    'lt': '(({0} < {1}) ? 1.0f : 0.0f)', 'gt': '(({0} > {1}) ? 1.0f : 0.0f)',
+    'le': '(({0} <= {1}) ? 1.0f : 0.0f)', 'ge': '(({0} >= {1}) ? 1.0f : 0.0f)',
+    'eq': '(({0} == {1}) ? 1.0f : 0.0f)', 'ne': '(({0} != {1}) ? 1.0f : 0.0f)',
+    'maximum': 'fmaxf({0}, {1})', 'minimum': 'fminf({0}, {1})',
+}
+
+
+def _dims(ext, R, C):
+    return (R if ext[0] else 1, C if ext[1] else 1)
+
+
+def _ref(name, ext, R, C, const):
+    rr, cc = _dims(ext, R, C)
+    return f"{'const ' if const else ''}float (&{name})[{rr}][{cc}]"
+
+
+def _at(name, ext):
+    return f"{name}[{'r' if ext[0] else '0'}][{'c' if ext[1] else '0'}]"
+
+
+def _loops(rr, cc):
+    return (f'#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
+            f'#pragma unroll\n  for (int c = 0; c < {cc}; c++)\n    ')
+
+
+def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple[bool, bool]],
+                  reduce_fn: str) -> Tuple[str, List[str]]:
+    """Device function evaluating `g` on register tiles.  Every value is a `float[RR][CC]`
+    array with RR = R if it varies along rows else 1, CC likewise for columns.  Returns the
+    source and the list of graph inputs that appear in the signature (the used ones)."""
+    ext = g.ext_table()
+    used = [i for i, u in zip(g.inputs, g.used_inputs()) if u]
+    params = [_ref(i, g.input_ext[i], R, C, True) for i in used]
+    params += [_ref(f'o{k}_', e, R, C, False) for k, e in enumerate(out_exts)]
+    out = [f'__device__ __forceinline__ void {fname}(' + ', '.join(params) + ') {']
+    for n in g.nodes:
+        rr, cc = _dims(n.ext, R, C)
+        out.append(f'  float {n.name}[{rr}][{cc}];')
+
+        def opnd(a):
+            return _at(a, ext[a]) if isinstance(a, str) else _lit(a)
+
+        if n.op == 'sum':
+            assert n.dims == (1,), n
+            src = n.args[0]
+            sext = ext[src]
+            assert sext[1]
+            srr = R if sext[0] else 1
+            s_at = f"{src}[{'r' if sext[0] else '0'}]"
+            out.append(f'#pragma unroll\n  for (int r = 0; r < {srr}; r++) {{\n'
+                       f'    float s_ = {s_at}[0];\n'
+                       f'#pragma unroll\n    for (int c = 1; c < {C}; c++) s_ += {s_at}[c];\n'
+                       f'    {n.name}[r][0] = {reduce_fn}(s_);\n  }}')
+        elif n.op == 'const':
+            out.append(f'  {n.name}[0][0] = {_lit(n.args[0])};')
+        elif n.op in _UNARY_EXPR:
+            out.append('  ' + _loops(rr, cc) + f'{n.name}[r][c] = ' + _UNARY_EXPR[n.op].format(opnd(n.args[0])) + ';')
+        elif n.op in _BINARY_EXPR:
+            out.append('  ' + _loops(rr, cc) + f'{n.name}[r][c] = '
+                       + _BINARY_EXPR[n.op].format(opnd(n.args[0]), opnd(n.args[1])) + ';')
+        elif n.op == 'where':
+            out.append('  ' + _loops(rr, cc) + f'{n.name}[r][c] = (({opnd(n.args[0])} != 0.0f) ? '
+                       f'{opnd(n.args[1])} : {opnd(n.args[2])});')
+        else:
+            raise NotImplementedError(n.op)
+    for k, (o, e) in enumerate(zip(g.outputs, out_exts)):
+        oe = ext[o]
+        assert (not oe[0] or e[0]) and (not oe[1] or e[1]), (fname, o, oe, e)
+        rr, cc = _dims(e, R, C)
+        out.append('  ' + _loops(rr, cc) + f'o{k}_[r][c] = {_at(o, oe)};')
+    out.append('}')
+    return '\n'.join(out), used
+
+
+# ------------------------------------------------------------------------------------ kernels
+
+@dataclass
+class KernelSpec:
+    name: str
+    source: str
+    tensors: List[str]          # logical tensor names, in Args order
+    block: int
+    grid: Tuple[str, str, str]  # python expressions over B, T, H, M, nch
+
+
+class _Args:
+    """Allocates TArg slots and renders `A.t[k]` accessors."""
+
+    def __init__(self):
+        self.names: List[str] = []
+
+    def slot(self, name: str) -> int:
+        if name not in self.names:
+            self.names.append(name)
+        return self.names.index(name)
+
+    def p(self, name: str) -> str:
+        return f'A.t[{self.slot(name)}].p'
+
+    def s(self, name: str, d: int) -> str:
+        return f'A.t[{self.slot(name)}].s[{d}]'
+
+    def struct(self) -> str:
+        return f'struct Args {{ TArg t[{max(len(self.names), 1)}]; int B, T, H, M, nch; }};\n'
+
+
+def _col_expr(C: int, L: int) -> str:
+    """Column owned by (lane-in-group l, element c).  With C >= 4 a lane owns float4
+    pieces, interleaved across the group so that 16 lanes x 16 B is one contiguous row
+    segment (conflict-free ds_read_b128, full-line global access)."""
+    if C >= 4:
+        return f'(((c) >> 2) * {4 * L} + l * 4 + ((c) & 3))'
+    return f'(l * {C} + (c))'
+
+
+class Emitter:
+    def __init__(self, plan):
+        self.plan = plan
+        self.p = plan.part
+        self.tile = plan.tile
+        p = self.p
+        self.cls = plan.in_cls
+        self.tdep = [not b[1] and plan.T > 1 for b in plan.in_bcast]      # varies with time
+        # an input with T == 1 overall is handled as time-dependent with a single step
+        self.tdep = [(plan.T == 1 or not b[1]) and c != 'mat' for b, c in zip(plan.in_bcast, self.cls)]
+        self.atomic = set(plan.atomic)
+        self.jext = p.joint.ext_table()
+
+    # ------------------------------------------------------------------ helpers
+    def in_ext(self, i: int):
+        return {'scalar': (False, False), 'col': (True, False), 'row': (False, True), 'mat': (True, True)}[self.cls[i]]
+
+    def _in_index(self, A: _Args, i: int, b='b', t='t', h='h', m=None, n=None) -> str:
+        """Element offset into input i (strides of broadcast dims are 0 at launch)."""
+        nm = f'in{i}'
+        terms = [f'(i64){b} * {A.s(nm, 0)}', f'(i64)({t}) * {A.s(nm, 1)}', f'(i64){h} * {A.s(nm, 2)}']
+        if m is not None:
+            terms.append(f'(i64)({m}) * {A.s(nm, 3)}')
+        if n is not None:
+            terms.append(f'(i64)({n}) * {A.s(nm, 4)}')
+        return ' + '.join(terms)
+
+    # ------------------------------------------------------------------ row kernels
+    def _row_kernel_common(self, A: _Args, used_inputs: List[int], R: int, W: int):
+        """Declarations shared by fw and bw1: thread mapping and staging buffers."""
+        t = self.tile
+        L, C, G = t.L, t.C, t.G
+        MT = W * G * R
+        N = self.plan.N
+        src = []
+        src.append(f'''  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l = lane % {L}, grp = lane / {L};
+  const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
+  const int rloc = (wave * {G} + grp) * {R};
+  const int row0 = mt * {MT} + rloc;
+  const int T = A.T, H = A.H, M = A.M, nch = A.nch;
+  (void)T; (void)H; (void)nch;
+#define COL(c) {_col_expr(C, L)}
+#define ROWC(r) (min(row0 + (r), M - 1))
+''')
+        return src, MT
+
+    def _stage_decl(self, nm: str, ext, TS: int, MT: int) -> str:
+        N = self.plan.N
+        ln = (N if ext[1] else 1) if not ext[0] else MT
+        return f'  __shared__ float {nm}[{TS}][{ln}];\n'
+
+    def _stage_in(self, A: _Args, i: int, TS: int, MT: int, NT: int, t0: str) -> str:
+        """Cooperative global -> LDS copy of input i for timesteps [t0, t0+TS)."""
+        ext = self.in_ext(i)
+        N = self.plan.N
+        dt = DT_CODE[self.plan.in_dtypes[i]]
+        if ext == (False, True):
+            ln, idx = N, self._in_index(A, i, t=f'{t0} + tt_', n='x_')
+            guard = ''
+        elif ext == (True, False):
+            ln, idx = MT, self._in_index(A, i, t=f'{t0} + tt_', m=f'min(mt * {MT} + x_, M - 1)')
+            guard = ''
+        else:
+            ln, idx = 1, self._in_index(A, i, t=f'{t0} + tt_')
+            guard = ''
+        return (f'    for (int e_ = tid; e_ < {TS * ln}; e_ += {NT}) {{ int tt_ = e_ / {ln}, x_ = e_ % {ln}; (void)x_;\n'
+                f'      s_in{i}[tt_][x_] = ldf<{dt}>({A.p(f"in{i}")}, {idx}); }}\n')
+
+    def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str) -> str:
+        """Registers <- staged LDS operand for timestep tt."""
+        rr, cc = _dims(ext, R, C)
+        if ext == (False, True):
+            return (f'      float {var}[1][{C}];\n#pragma unroll\n      for (int c = 0; c < {C}; c++) '
+                    f'{var}[0][c] = {sname}[{tt}][COL(c)];\n')
+        if ext == (True, False):
+            return (f'      float {var}[{R}][1];\n#pragma unroll\n      for (int r = 0; r < {R}; r++) '
+                    f'{var}[r][0] = {sname}[{tt}][rloc + r];\n')
+        if ext == (False, False):
+            return f'      float {var}[1][1]; {var}[0][0] = {sname}[{tt}][0];\n'
+        raise AssertionError
+
+    def _load_const_input(self, A: _Args, i: int, R: int, C: int) -> str:
+        """Time-independent input -> registers, once."""
+        ext = self.in_ext(i)
+        rr, cc = _dims(ext, R, C)
+        dt = DT_CODE[self.plan.in_dtypes[i]]
+        idx = self._in_index(A, i, t='0', m='ROWC(r)' if ext[0] else None, n='COL(c)' if ext[1] else None)
+        return (f'  float x{i}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
+                f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) x{i}[r][c] = ldf<{dt}>({A.p(f"in{i}")}, {idx});\n')
+
+    def _ck_index(self, chunk: str) -> str:
+        N = self.plan.N
+        return f'(((i64)(b * H + h) * nch + ({chunk})) * M + (row0 + r)) * {N} + COL(c)'
+
+    # ------------------------------------------------------------------ fw
+    def fw(self) -> KernelSpec:
+        p, plan, t = self.p, self.plan, self.tile
+        L, C, G, R, W, DT, TS = t.L, t.C, t.G, t.R, t.W, t.DT, t.TS
+        N = plan.N
+        NT = W * 64
+        A = _Args()
+        g = p.fw
+        nin, nst, nout, naux = p.ninputs, p.nstates, p.noutputs, len(p.aux)
+        out_exts = [(True, False)] * nout + [(True, True)] * nst + [(True, False)] * naux
+        # a state of a problem with M == 1 or N == 1 has a smaller extent; follow the joint graph
+        st_ext = [self.jext[s] for s in p.st_names]
+        out_exts = [(st_ext[0][0], False)] * nout + st_ext + [(st_ext[0][0], False)] * naux
+        fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>')
+        used_in = [i for i in range(nin) if p.in_names[i] in used]
+        src, MT = self._row_kernel_common(A, used_in, R, W)
+        body = []
+        # staging buffers
+        for i in used_in:
+            if self.tdep[i]:
+                body.append(self._stage_decl(f's_in{i}', self.in_ext(i), TS, MT))
+        for k in range(nout):
+            body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
+        for k in range(naux):
+            body.append(f'  __shared__ float s_aux{k}[{TS}][{MT}];\n')
+        # state
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            dt = DT_CODE[plan.st_dtypes[k]]
+            nm = f'st{k}'
+            body.append(f'  float S{k}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
+                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) S{k}[r][c] = ldf<{dt}>({A.p(nm)}, '
+                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)ROWC(r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)});\n')
+        for i in used_in:
+            if not self.tdep[i]:
+                body.append(self._load_const_input(A, i, R, C))
+        body.append(f'  for (int t0 = 0; t0 < T; t0 += {TS}) {{\n')
+        # checkpoint
+        body.append(f'    if (t0 % {DT} == 0) {{\n')
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                        f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
+                        f'((float*){A.p(f"sck{k}")})[{self._ck_index(f"t0 / {DT}")}] = S{k}[r][c]; }}\n')
+        body.append('    }\n    __syncthreads();\n')
+        for i in used_in:
+            if self.tdep[i]:
+                body.append(self._stage_in(A, i, TS, MT, NT, 't0'))
+        body.append('    __syncthreads();\n')
+        body.append(f'#pragma unroll 2\n    for (int tt = 0; tt < {TS}; tt++) {{\n')
+        call = []
+        for nm_ in used:
+            if nm_ in p.in_names:
+                i = p.in_names.index(nm_)
+                if self.tdep[i]:
+                    body.append(self._load_operand(f'x{i}', f's_in{i}', self.in_ext(i), R, C, 'tt'))
+                call.append(f'x{i}')
+            elif nm_ in p.st_names:
+                call.append(f'S{p.st_names.index(nm_)}')
+            else:
+                raise AssertionError(nm_)
+        rrs = R if st_ext[0][0] else 1
+        for k in range(nout):
+            body.append(f'      float y{k}[{rrs}][1];\n')
+            call.append(f'y{k}')
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'      float nS{k}[{rr}][{cc}];\n')
+            call.append(f'nS{k}')
+        for k in range(naux):
+            body.append(f'      float a{k}[{rrs}][1];\n')
+            call.append(f'a{k}')
+        body.append('      fw_step(' + ', '.join(call) + ');\n')
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++)\n#pragma unroll\n      for (int c = 0; c < {cc}; c++) S{k}[r][c] = nS{k}[r][c];\n')
+        body.append('      if (l == 0) {\n')
+        for k in range(nout):
+            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_out{k}[tt][rloc + r] = y{k}[{"r" if rrs > 1 else "0"}][0];\n')
+        for k in range(naux):
+            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_aux{k}[tt][rloc + r] = a{k}[{"r" if rrs > 1 else "0"}][0];\n')
+        body.append('      }\n    }\n    __syncthreads();\n')
+        # flush
+        body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
+                    f'      if (m_ < M) {{\n')
+        for k in range(nout):
+            dt = DT_CODE[plan.out_dtypes[k]]
+            nm = f'out{k}'
+            body.append(f'        stf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}, s_out{k}[tt_][x_]);\n')
+        for k in range(naux):
+            body.append(f'        ((float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_] = s_aux{k}[tt_][x_];\n')
+        body.append('      } }\n  }\n')
+        # final state
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            dt = DT_CODE[plan.st_dtypes[k]]
+            nm = f'stT{k}'
+            body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) stf<{dt}>({A.p(nm)}, '
+                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, S{k}[r][c]); }}\n')
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_fw(Args A) {{\n'
+                  + ''.join(src) + ''.join(body) + '}\n')
+        source = PRELUDE + A.struct() + fn_src + '\n' + kernel
+        return KernelSpec('frnn_fw', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
+
+    # ------------------------------------------------------------------ bw1
+    def bw1(self) -> KernelSpec:
+        p, plan, t = self.p, self.plan, self.tile
+        L, C, G, DT = t.L, t.C, t.G, t.DT
+        R, W = (t.R1 or t.R), (t.W1 or t.W)
+        needs_state = p.dstep_needs_state
+        TS = DT if needs_state else t.TS
+        N = plan.N
+        NT = W * 64
+        A = _Args()
+        nin, nst, nout = p.ninputs, p.nstates, p.noutputs
+        naux, ndaux = len(p.aux), len(p.daux)
+        st_ext = [self.jext[s] for s in p.st_names]
+        colx = (st_ext[0][0], False)
+        rrs = R if colx[0] else 1
+        g = p.dstep
+        out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux
+        fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>')
+        fns = [fn_src]
+        used_all = set(used)
+        re_used = []
+        if needs_state:
+            re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>')
+            fns.append(re_src)
+            used_all |= set(re_used)
+        used_in = [i for i in range(nin) if p.in_names[i] in used_all]
+        used_aux = [k for k in range(naux) if p.aux[k] in used_all]
+        used_dout = [k for k in range(nout) if p.dout_names[k] in used_all]
+        src, MT = self._row_kernel_common(A, used_in, R, W)
+        body = []
+        for i in used_in:
+            if self.tdep[i]:
+                body.append(self._stage_decl(f's_in{i}', self.in_ext(i), TS, MT))
+        for k in used_aux:
+            body.append(f'  __shared__ float s_aux{k}[{TS}][{MT}];\n')
+        for k in used_dout:
+            body.append(f'  __shared__ float s_dy{k}[{TS}][{MT}];\n')
+        tdep_col = [i for i in p.col_idx if self.tdep[i]]
+        const_col = [i for i in p.col_idx if not self.tdep[i]]
+        for i in tdep_col:
+            body.append(f'  __shared__ float s_dc{i}[{TS}][{MT}];\n')
+        for k in range(ndaux):
+            body.append(f'  __shared__ float s_da{k}[{TS}][{MT}];\n')
+        # incoming cotangent of the final state
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            dt = DT_CODE[plan.st_dtypes[k]]
+            nm = f'dstT{k}'
+            body.append(f'  float D{k}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
+                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) D{k}[r][c] = ldf<{dt}>({A.p(nm)}, '
+                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)ROWC(r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)});\n')
+        for i in used_in:
+            if not self.tdep[i]:
+                body.append(self._load_const_input(A, i, R, C))
+        for i in const_col:
+            body.append(f'  float gacc{i}[{rrs}][1];\n#pragma unroll\n  for (int r = 0; r < {rrs}; r++) gacc{i}[r][0] = 0.0f;\n')
+        body.append(f'  for (int t0 = T - {TS}; t0 >= 0; t0 -= {TS}) {{\n')
+        body.append(f'    if ((t0 + {TS}) % {DT} == 0) {{\n')
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                        f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
+                        f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"(t0 + {TS}) / {DT} - 1")}] = D{k}[r][c]; }}\n')
+        body.append('    }\n    __syncthreads();\n')
+        for i in used_in:
+            if self.tdep[i]:
+                body.append(self._stage_in(A, i, TS, MT, NT, 't0'))
+        stage_rows = (f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; '
+                      f'int m_ = min(mt * {MT} + x_, M - 1);\n')
+        if used_aux or used_dout:
+            body.append(stage_rows)
+            for k in used_aux:
+                body.append(f'      s_aux{k}[tt_][x_] = ((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_];\n')
+            for k in used_dout:
+                dt = DT_CODE[plan.out_dtypes[k]]
+                nm = f'dout{k}'
+                body.append(f'      s_dy{k}[tt_][x_] = ldf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)});\n')
+            body.append('    }\n')
+        body.append('    __syncthreads();\n')
+
+        def operand_loads(tt, names, state_var):
+            code, call = [], []
+            for nm_ in names:
+                if nm_ in p.in_names:
+                    i = p.in_names.index(nm_)
+                    if self.tdep[i]:
+                        code.append(self._load_operand(f'x{i}_{tt}' if needs_state else f'x{i}', f's_in{i}', self.in_ext(i), R, C, tt))
+                        call.append(f'x{i}_{tt}' if needs_state else f'x{i}')
+                    else:
+                        call.append(f'x{i}')
+                elif nm_ in p.st_names:
+                    call.append(state_var(p.st_names.index(nm_)))
+                elif nm_ in p.aux:
+                    k = p.aux.index(nm_)
+                    e = self.jext[nm_]
+                    v = f'ax{k}_{tt}' if needs_state else f'ax{k}'
+                    code.append(self._load_operand(v, f's_aux{k}', (e[0], False), R, C, tt))
+                    call.append(v)
+                elif nm_ in p.dout_names:
+                    k = p.dout_names.index(nm_)
+                    v = f'dy{k}_{tt}' if needs_state else f'dy{k}'
+                    code.append(self._load_operand(v, f's_dy{k}', colx, R, C, tt))
+                    call.append(v)
+                elif nm_ in p.dnst_names:
+                    call.append(f'D{p.dnst_names.index(nm_)}')
+                else:
+                    raise AssertionError(nm_)
+            return code, call
+
+        def dstep_block(tt, state_var, indent='      '):
+            code, call = operand_loads(tt, used, state_var)
+            for k in range(nst):
+                rr, cc = _dims(st_ext[k], R, C)
+                code.append(f'{indent}float nD{k}[{rr}][{cc}];\n')
+                call.append(f'nD{k}')
+            for i in p.col_idx:
+                code.append(f'{indent}float gc{i}[{rrs}][1];\n')
+                call.append(f'gc{i}')
+            for k in range(ndaux):
+                code.append(f'{indent}float da{k}[{rrs}][1];\n')
+                call.append(f'da{k}')
+            code.append(f'{indent}bw_dstep(' + ', '.join(call) + ');\n')
+            for k in range(nst):
+                rr, cc = _dims(st_ext[k], R, C)
+                code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {rr}; r++)\n#pragma unroll\n{indent}for (int c = 0; c < {cc}; c++) D{k}[r][c] = nD{k}[r][c];\n')
+            for i in const_col:
+                code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {rrs}; r++) gacc{i}[r][0] += gc{i}[r][0];\n')
+            code.append(f'{indent}if (l == 0) {{\n')
+            ridx = 'r' if rrs > 1 else '0'
+            for i in tdep_col:
+                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_dc{i}[{tt}][rloc + r] = gc{i}[{ridx}][0];\n')
+            for k in range(ndaux):
+                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_da{k}[{tt}][rloc + r] = da{k}[{ridx}][0];\n')
+            code.append(f'{indent}}}\n')
+            return code
+
+        if not needs_state:
+            body.append(f'#pragma unroll 2\n    for (int tt = {TS - 1}; tt >= 0; tt--) {{\n')
+            body += dstep_block('tt', lambda k: (_ for _ in ()).throw(AssertionError()))
+            body.append('    }\n')
+        else:
+            # recompute the DT states of this chunk from its checkpoint, then walk back
+            for k in range(nst):
+                rr, cc = _dims(st_ext[k], R, C)
+                body.append(f'    float Sh{k}_0[{rr}][{cc}];\n#pragma unroll\n    for (int r = 0; r < {rr}; r++)\n'
+                            f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = '
+                            f'((const float*){A.p(f"sck{k}")})[(((i64)(b * H + h) * nch + (t0 / {DT})) * M + ROWC(r)) * {N} + COL(c)];\n')
+            for tt in range(1, DT):
+                for k in range(nst):
+                    rr, cc = _dims(st_ext[k], R, C)
+                    body.append(f'    float Sh{k}_{tt}[{rr}][{cc}];\n')
+            for tt in range(DT - 1):
+                body.append('    {\n')
+                code, call = operand_loads(str(tt), re_used, lambda k, tt=tt: f'Sh{k}_{tt}')
+                body += code
+                for k in range(nst):
+                    call.append(f'Sh{k}_{tt + 1}')
+                body.append('      bw_restep(' + ', '.join(call) + ');\n    }\n')
+            for tt in range(DT - 1, -1, -1):
+                body.append('    {\n')
+                body += dstep_block(str(tt), lambda k, tt=tt: f'Sh{k}_{tt}')
+                body.append('    }\n')
+        body.append('    __syncthreads();\n')
+        # flush column grads and daux
+        if tdep_col or ndaux:
+            body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
+                        f'      if (m_ < M) {{\n')
+            for i in tdep_col:
+                nm = f'din{i}'
+                idx = f'(i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}'
+                if i in self.atomic:
+                    body.append(f'        atomic_addf({A.p(nm)}, {idx}, s_dc{i}[tt_][x_]);\n')
+                else:
+                    dt = DT_CODE[plan.in_dtypes[i]]
+                    body.append(f'        stf<{dt}>({A.p(nm)}, {idx}, s_dc{i}[tt_][x_]);\n')
+            for k in range(ndaux):
+                body.append(f'        ((float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_] = s_da{k}[tt_][x_];\n')
+            body.append('      } }\n')
+        body.append('  }\n')
+        for i in const_col:
+            nm = f'din{i}'
+            body.append(f'  if (l == 0) {{\n#pragma unroll\n    for (int r = 0; r < {R}; r++) if (row0 + r < M) '
+                        f'atomic_addf({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 2)} + (i64)(row0 + r) * {A.s(nm, 3)}, gacc{i}[{"r" if rrs > 1 else "0"}][0]);\n  }}\n')
+        for k in range(nst):
+            rr, cc = _dims(st_ext[k], R, C)
+            dt = DT_CODE[plan.st_dtypes[k]]
+            nm = f'dst{k}'
+            body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) stf<{dt}>({A.p(nm)}, '
+                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, D{k}[r][c]); }}\n')
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw1(Args A) {{\n'
+                  + ''.join(src) + ''.join(body) + '}\n')
+        source = PRELUDE + A.struct() + '\n'.join(fns) + '\n' + kernel
+        return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
+
+    # ------------------------------------------------------------------ bw2
+    def bw2(self) -> KernelSpec:
+        p, plan, t = self.p, self.plan, self.tile
+        N, DT = plan.N, t.DT
+        IPB = max(1, 64 // N)
+        NT = max(64, N)
+        A = _Args()
+        nin, nst, nout = p.ninputs, p.nstates, p.noutputs
+        naux, ndaux = len(p.aux), len(p.daux)
+        st_ext = [self.jext[s] for s in p.st_names]
+        nm_ = p.joint.node_map()
+        rs = p.row_idx + p.scalar_idx
+        red = f'inst_allreduce<{N}>'
+        op_names = [nm_[m].args[0] for m in p.msums]
+        drow_exts = st_ext + [(True, True)] * len(p.mat_idx) + [self.jext[o] for o in op_names]
+        drow_src, drow_used = emit_graph_fn(p.drow, 'bw_drow', 1, 1, drow_exts, red)
+        re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', 1, 1, st_ext, red)
+        epi_exts = [self.in_ext(i) for i in rs]
+        epi_src, epi_used = emit_graph_fn(p.epi, 'bw_epi', 1, 1, epi_exts, red)
+        loop_used = set(drow_used) | set(re_used)
+        all_used = loop_used | set(epi_used)
+
+        def is_rowlike(nm):      # no row extent: can be loaded once per chunk
+            return not self.jext[nm][0]
+
+        helper = f'''
+template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
+  if constexpr (N_ <= 64) {{ return grp_allreduce<N_>(x); }}
+  else {{
+    __shared__ float red_[N_ / 64];
+    x = grp_allreduce<64>(x);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) red_[threadIdx.x >> 6] = x;
+    __syncthreads();
+    float s = 0.0f;
+#pragma unroll
+    for (int w = 0; w < N_ / 64; w++) s += red_[w];
+    return s;
+  }}
+}}
+'''
+        b = []
+        b.append(f'''  const int tid = threadIdx.x;
+  const int n = tid % {N};
+  const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
+  const int T = A.T, H = A.H, M = A.M, nch = A.nch;
+  (void)T;
+  int ch = blockIdx.x * {IPB} + inst;
+  const bool valid = ch < nch;
+  if (!valid) ch = nch - 1;
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const int t0 = ch * {DT};
+''')
+
+        def load_in(i, tt, m=None):
+            ext = self.in_ext(i)
+            dt = DT_CODE[plan.in_dtypes[i]]
+            idx = self._in_index(A, i, t=(f't0 + {tt}' if self.tdep[i] else '0'),
+                                 m=('m' if ext[0] else None), n=('n' if ext[1] else None))
+            return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
+
+        def var_in(i, tt):
+            return f'x{i}_{tt}' if self.tdep[i] else f'x{i}'
+
+        def aux_load(k, tt, mexpr):
+            return f'((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + {mexpr}]'
+
+        def daux_load(k, tt):
+            return f'((const float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + m]'
+
+        def dy_load(k, tt):
+            dt = DT_CODE[plan.out_dtypes[k]]
+            nmv = f'dout{k}'
+            return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)(t0 + {tt}) * {A.s(nmv, 1)} + '
+                    f'(i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)})')
+
+        # ---- per-chunk loads of everything without a row extent
+        for i in range(nin):
+            if p.in_names[i] not in all_used or self.in_ext(i)[0]:
+                continue
+            if self.tdep[i]:
+                for tt in range(DT):
+                    b.append(f'  float x{i}_{tt}[1][1]; x{i}_{tt}[0][0] = {load_in(i, tt)};\n')
+            else:
+                b.append(f'  float x{i}[1][1]; x{i}[0][0] = {load_in(i, 0)};\n')
+        for k in range(naux):
+            if p.aux[k] in all_used and is_rowlike(p.aux[k]):
+                for tt in range(DT):
+                    b.append(f'  float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "0")};\n')
+        for j in range(len(p.msums)):
+            for tt in range(DT):
+                b.append(f'  float acc{j}_{tt} = 0.0f;\n')
+        # ---- row loop
+        b.append('  for (int m = 0; m < M; m++) {\n')
+        b.append(f'    const i64 cko = (((i64)bh * nch + ch) * M + m) * {N} + n;\n')
+        for k in range(nst):
+            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = ((const float*){A.p(f"sck{k}")})[cko];\n')
+            b.append(f'    float D{k}[1][1]; D{k}[0][0] = ((const float*){A.p(f"dck{k}")})[cko];\n')
+        for i in range(nin):
+            if p.in_names[i] not in loop_used or not self.in_ext(i)[0]:
+                continue
+            if self.tdep[i]:
+                for tt in range(DT):
+                    b.append(f'    float x{i}_{tt}[1][1]; x{i}_{tt}[0][0] = {load_in(i, tt)};\n')
+            else:
+                b.append(f'    float x{i}[1][1]; x{i}[0][0] = {load_in(i, 0)};\n')
+        for k in range(naux):
+            if p.aux[k] in loop_used and not is_rowlike(p.aux[k]):
+                for tt in range(DT):
+                    b.append(f'    float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "m")};\n')
+        for k in range(ndaux):
+            if p.daux[k] in loop_used:
+                for tt in range(DT):
+                    b.append(f'    float da{k}_{tt}[1][1]; da{k}_{tt}[0][0] = {daux_load(k, tt)};\n')
+        for k in range(nout):
+            if p.dout_names[k] in loop_used:
+                for tt in range(DT):
+                    b.append(f'    float dy{k}_{tt}[1][1]; dy{k}_{tt}[0][0] = {dy_load(k, tt)};\n')
+
+        def call_args(names, tt, state_var):
+            call = []
+            for v in names:
+                if v in p.in_names:
+                    call.append(var_in(p.in_names.index(v), tt))
+                elif v in p.st_names:
+                    call.append(state_var(p.st_names.index(v)))
+                elif v in p.aux:
+                    call.append(f'ax{p.aux.index(v)}_{tt}')
+                elif v in p.daux:
+                    call.append(f'da{p.daux.index(v)}_{tt}')
+                elif v in p.dout_names:
+                    call.append(f'dy{p.dout_names.index(v)}_{tt}')
+                elif v in p.dnst_names:
+                    call.append(f'D{p.dnst_names.index(v)}')
+                elif v in p.msums:
+                    call.append(f'ms{p.msums.index(v)}')
+                else:
+                    raise AssertionError(v)
+            return call
+
+        for tt in range(DT - 1):
+            for k in range(nst):
+                b.append(f'    float Sh{k}_{tt + 1}[1][1];\n')
+            call = call_args(re_used, tt, lambda k, tt=tt: f'Sh{k}_{tt}') + [f'Sh{k}_{tt + 1}' for k in range(nst)]
+            b.append('    bw_restep(' + ', '.join(call) + ');\n')
+        for i in p.mat_idx:
+            b.append(f'    float ma{i} = 0.0f;\n')
+        for tt in range(DT - 1, -1, -1):
+            b.append('    {\n')
+            call = call_args(drow_used, tt, lambda k, tt=tt: f'Sh{k}_{tt}')
+            for k in range(nst):
+                b.append(f'      float nD{k}[1][1];\n')
+                call.append(f'nD{k}')
+            for i in p.mat_idx:
+                b.append(f'      float gm{i}[1][1];\n')
+                call.append(f'gm{i}')
+            for j in range(len(p.msums)):
+                b.append(f'      float op{j}[1][1];\n')
+                call.append(f'op{j}')
+            b.append('      bw_drow(' + ', '.join(call) + ');\n')
+            for k in range(nst):
+                b.append(f'      D{k}[0][0] = nD{k}[0][0];\n')
+            for i in p.mat_idx:
+                b.append(f'      ma{i} += gm{i}[0][0];\n')
+            for j in range(len(p.msums)):
+                b.append(f'      acc{j}_{tt} += op{j}[0][0];\n')
+            b.append('    }\n')
+        for i in p.mat_idx:
+            nmv = f'din{i}'
+            idx = f'(i64)b * {A.s(nmv, 0)} + (i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)} + (i64)n * {A.s(nmv, 4)}'
+            b.append(f'    if (valid) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
+        b.append('  }\n')
+        # ---- epilogue
+        for tt in range(DT):
+            b.append('  {\n')
+            for j, mname in enumerate(p.msums):
+                node = nm_[mname]
+                opext = self.jext[node.args[0]]
+                if 1 in node.dims and opext[1]:
+                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}(acc{j}_{tt});\n')
+                else:
+                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = acc{j}_{tt};\n')
+            call = call_args(epi_used, tt, None)
+            for i in rs:
+                b.append(f'    float g{i}[1][1];\n')
+                call.append(f'g{i}')
+            b.append('    bw_epi(' + ', '.join(call) + ');\n')
+            for i in rs:
+                nmv = f'din{i}'
+                ext = self.in_ext(i)
+                tterm = f'(i64)(t0 + {tt}) * {A.s(nmv, 1)}'
+                idx = f'(i64)b * {A.s(nmv, 0)} + {tterm} + (i64)h * {A.s(nmv, 2)}' + (f' + (i64)n * {A.s(nmv, 4)}' if ext[1] else '')
+                cond = 'valid' + ('' if ext[1] else ' && n == 0')
+                if i in self.atomic:
+                    b.append(f'    if ({cond}) atomic_addf({A.p(nmv)}, {idx}, g{i}[0][0]);\n')
+                else:
+                    dt = DT_CODE[plan.in_dtypes[i]]
+                    b.append(f'    if ({cond}) stf<{dt}>({A.p(nmv)}, {idx}, g{i}[0][0]);\n')
+            b.append('  }\n')
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
+        source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + kernel
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', 'B * H', '1'))

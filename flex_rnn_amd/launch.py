@@ -1,0 +1,128 @@
+"""Host side of the compiled path: builds the three kernels of a plan through the C-ABI
+runtime, allocates results / hidden buffers with torch, packs the kernel argument block
+and launches on torch's current stream.
+
+Counterpart of the reference's `forward` / `backward` closures
+(/root/reference/flex_rnn/twopass.py:224-237, 343-363): same buffers in the same order
+(outputs, final states, state checkpoints, packed aux | input grads, initial-state grads),
+fp32 scratch + cast-back for gradients of inputs broadcast over batch / time / head
+(twopass.py:181, 355, 359-360).  There is no CPU execution path here.
+"""
+from __future__ import annotations
+
+import struct
+from typing import Dict, List, Sequence, Tuple
+
+import torch as th
+
+from . import runtime
+from .emit_hip import Emitter, KernelSpec
+
+
+def _strides5(t: th.Tensor) -> Tuple[int, ...]:
+    s = [st if n > 1 else 0 for st, n in zip(t.stride(), t.shape)]
+    return tuple(s + [0] * (5 - len(s)))
+
+
+def kernel_specs(plan) -> List[KernelSpec]:
+    em = Emitter(plan)
+    return [em.fw(), em.bw1(), em.bw2()]
+
+
+def compile_plan(plan, force: bool = False) -> List[Tuple[KernelSpec, str]]:
+    """Emit + compile (or fetch from the cache) the three kernels.  Needs no GPU."""
+    return [(s, runtime.compile_kernel(s.name, s.source, force=force)) for s in kernel_specs(plan)]
+
+
+class CompiledPlan:
+    def __init__(self, plan, state_meta=None):
+        self.plan = plan
+        # (shape, stride, dtype) of the initial states: gradients w.r.t. them are laid out alike
+        self.state_meta = state_meta
+        built = compile_plan(plan)
+        self.kernels = {}
+        self.modules = []
+        for spec, path in built:
+            mod = runtime.Module(path)
+            self.modules.append(mod)
+            self.kernels[spec.name] = (spec, mod.kernel(spec.name))
+
+    # ------------------------------------------------------------------ launch helper
+    def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
+        spec, kern = self.kernels[kname]
+        pl = self.plan
+        buf = bytearray()
+        dev = None
+        for name in spec.tensors:
+            t = tensors[name]
+            assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
+            dev = t.device if dev is None else dev
+            assert t.device == dev, 'all tensors must live on the same device'
+            buf += struct.pack('<q5q', t.data_ptr(), *_strides5(t))
+        if not spec.tensors:
+            buf += struct.pack('<q5q', 0, 0, 0, 0, 0, 0)
+        buf += struct.pack('<5i', pl.B, pl.T, pl.H, pl.M, pl.nchunks)
+        env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
+        grid = tuple(int(eval(g, {}, env)) for g in spec.grid)
+        with th.cuda.device(dev):
+            stream = th.cuda.current_stream(dev).cuda_stream
+            kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
+        pl, p = self.plan, self.plan.part
+        dev = inputs[0].device
+        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
+        outs = tuple(th.empty(B, T, H, M, dtype=dt, device=dev) for dt in pl.out_dtypes)
+        stT = tuple(th.empty_like(s) for s in state0)
+        sck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state0)
+        aux = th.empty(len(p.aux), B, H, T, M, dtype=th.float32, device=dev)
+        tensors = {'aux': aux}
+        for i, x in enumerate(inputs):
+            tensors[f'in{i}'] = x
+        for k in range(p.nstates):
+            tensors[f'st{k}'] = state0[k]
+            tensors[f'stT{k}'] = stT[k]
+            tensors[f'sck{k}'] = sck[k]
+        for k in range(p.noutputs):
+            tensors[f'out{k}'] = outs[k]
+        self._launch('frnn_fw', tensors)
+        return (*outs, *stT, *sck, aux)
+
+    # ------------------------------------------------------------------ backward
+    def backward(self, doutput, dstateT, inputs, state_store, aux):
+        pl, p = self.plan, self.plan.part
+        dev = inputs[0].device
+        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
+        atomic = set(pl.atomic)
+        daux = th.empty(len(p.daux), B, H, T, M, dtype=th.float32, device=dev)
+        dck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state_store)
+        if self.state_meta is not None:
+            dst0 = tuple(th.empty_strided(sh, st, dtype=dt, device=dev) for sh, st, dt in self.state_meta)
+        else:
+            dst0 = tuple(th.empty_like(s) for s in dstateT)
+        dins = []
+        for i, x in enumerate(inputs):
+            if i in atomic:
+                dins.append(th.zeros(x.shape, dtype=th.float32, device=dev))
+            else:
+                dins.append(th.empty_like(x))
+        tensors = {'aux': aux, 'daux': daux}
+        for i, x in enumerate(inputs):
+            tensors[f'in{i}'] = x
+            tensors[f'din{i}'] = dins[i]
+        for k in range(p.nstates):
+            tensors[f'dstT{k}'] = dstateT[k]
+            tensors[f'dst{k}'] = dst0[k]
+            tensors[f'sck{k}'] = state_store[k]
+            tensors[f'dck{k}'] = dck[k]
+        for k in range(p.noutputs):
+            tensors[f'dout{k}'] = doutput[k]
+        self._launch('frnn_bw1', tensors)
+        self._launch('frnn_bw2', tensors)
+        for i in atomic:
+            x = inputs[i]
+            g = th.empty_like(x)
+            g.copy_(dins[i])
+            dins[i] = g
+        return tuple(dins), dst0

@@ -1,0 +1,71 @@
+"""Ahead-of-time kernel cache warm-up.
+
+Kernels are normally compiled on the first call of a `jit` object; `warm()` runs the
+same planner + emitter + hipcc step for a list of workloads without a GPU, so that a
+machine without a compiler in the loop (or a test run) finds every code object in the
+cache.  `CASES` lists the workloads the test-suite, the smoke test and the benchmark use.
+"""
+from __future__ import annotations
+
+from typing import Iterable, List, Optional, Tuple
+
+import torch as th
+
+from . import configs, planner
+from .launch import compile_plan
+
+# (workload name, (B, T, H, M, N) or None for the full benchmark size, dtype or None)
+CASES: List[Tuple[str, Optional[tuple], Optional[th.dtype]]] = [
+    # reduced sizes used by the parity tests (same M, N as the full configurations)
+    ('delta_rule', None, None),
+    ('mamba1', (2, 64, 4, 128, 16), None),
+    ('mamba2', (2, 64, 4, 64, 128), None),
+    ('rwkv7', (2, 64, 2, 128, 128), None),
+    ('rwkv7', (2, 64, 2, 128, 128), th.float32),
+    ('gated_delta_rule', (2, 128, 2, 128, 128), None),
+    # full benchmark sizes
+    ('mamba1', None, None),
+    ('mamba2', None, None),
+    ('rwkv7', None, None),
+    ('gated_delta_rule', None, None),
+]
+
+
+def plan_for(name: str, dims=None, dtype=None, tile=None):
+    """Plan for a named workload built from meta tensors only (no data is generated)."""
+    dims = dims or configs.DEFAULT_DIMS[name]
+    small = configs.make(name, dims=(1, 1, 1, dims[3], dims[4]), dtype=dtype)
+    B, T, H, M, N = dims
+    full = (B, T, H, M, N)
+    ins = []
+    for x in small.inputs:
+        shape = tuple(full[j] if (x.shape[j] != 1 or _is_full(name, len(ins), j)) else 1 for j in range(5))
+        ins.append(th.empty(shape, dtype=x.dtype, device='meta'))
+    sts = [th.empty((B, H, M, N), dtype=s.dtype, device='meta') for s in small.states]
+    return planner.make_plan(small.step, ins, sts, tile)[0]
+
+
+# which of (B, T, H) each input of each workload spans (inputs built at B=T=H=1 lose that information)
+_SPANS = {
+    'delta_rule': ['BTH'] * 4,
+    'mamba1': ['BTH', 'BTH', 'H', 'BT', 'BT'],
+    'mamba2': ['BTH', 'BTH', 'H', 'BT', 'BT'],
+    'rwkv7': ['BTH'] * 6,
+    'gated_delta_rule': ['BTH'] * 5,
+}
+
+
+def _is_full(name: str, i: int, j: int) -> bool:
+    return j < 3 and 'BTH'[j] in _SPANS[name][i]
+
+
+def warm(cases: Iterable = CASES, verbose: bool = False, force: bool = False) -> int:
+    n = 0
+    done = set()
+    for name, dims, dtype in cases:
+        plan = plan_for(name, dims, dtype)
+        for spec, path in compile_plan(plan, force=force and (name, dims, dtype) not in done):
+            n += 1
+            if verbose:
+                print(f'  {name} {dims or "full"} {spec.name}: {path}')
+    return n

@@ -1,0 +1,156 @@
+"""ctypes binding of the C-ABI kernel runtime (`libfrnn_rt.so`, include/frnn_rt.h).
+
+`build_library()` compiles the runtime in-tree; `lib()` loads it and fails loudly
+when it has not been built.  `compile_kernel()` turns HIP source into a cached
+gfx950 code object (no GPU needed); `Module` / `Kernel` load and launch it.
+"""
+from __future__ import annotations
+
+import ctypes
+import hashlib
+import os
+import struct
+import subprocess
+from typing import Optional, Sequence, Tuple
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_ROOT = os.path.dirname(_HERE)
+LIB_PATH = os.path.join(_HERE, 'libfrnn_rt.so')
+ARCH = 'gfx950'
+EMITTER_OPTS = '-ffp-contract=fast -munsafe-fp-atomics'
+
+_lib = None
+
+
+class RuntimeError_(RuntimeError):
+    pass
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compile flex_rnn_amd/csrc/frnn_rt.cpp -> flex_rnn_amd/libfrnn_rt.so."""
+    src = os.path.join(_HERE, 'csrc', 'frnn_rt.cpp')
+    inc = os.path.join(_ROOT, 'include')
+    tmp = LIB_PATH + f'.tmp{os.getpid()}'
+    cmd = ['g++', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall', '-I', inc, src, '-o', tmp, '-ldl', '-pthread']
+    if verbose:
+        print(' '.join(cmd))
+    subprocess.run(cmd, check=True)
+    os.replace(tmp, LIB_PATH)
+    global _lib
+    _lib = None
+    return LIB_PATH
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.isfile(LIB_PATH):
+        raise RuntimeError_(
+            f'{LIB_PATH} is missing: the HIP kernel runtime has not been built. '
+            'Run `python -c "import __graft_entry__ as g; g.build()"` (or flex_rnn_amd.runtime.build_library()). '
+            'There is no CPU fallback for the compiled path; use `.naive` for a pure-PyTorch run.')
+    L = ctypes.CDLL(LIB_PATH)
+    L.frnn_version.restype = ctypes.c_int
+    L.frnn_last_error.restype = ctypes.c_char_p
+    L.frnn_compile.restype = ctypes.c_int
+    L.frnn_compile.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.c_char_p, ctypes.c_char_p,
+                               ctypes.c_char_p, ctypes.c_char_p, ctypes.c_char_p, ctypes.c_size_t]
+    L.frnn_module_load.restype = ctypes.c_int
+    L.frnn_module_load.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
+    L.frnn_get_kernel.restype = ctypes.c_int
+    L.frnn_get_kernel.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
+    L.frnn_launch.restype = ctypes.c_int
+    L.frnn_launch.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
+                              ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    L.frnn_module_free.restype = ctypes.c_int
+    L.frnn_module_free.argtypes = [ctypes.c_void_p]
+    L.frnn_device_cus.restype = ctypes.c_int
+    _lib = L
+    return L
+
+
+EXPORTS = ('frnn_version', 'frnn_last_error', 'frnn_compile', 'frnn_module_load', 'frnn_get_kernel',
+           'frnn_launch', 'frnn_module_free', 'frnn_device_cus')
+
+
+def _check(rc: int, what: str):
+    if rc != 0:
+        msg = lib().frnn_last_error().decode('utf-8', 'replace')
+        raise RuntimeError_(f'{what} failed (code {rc}): {msg}')
+
+
+def cache_dir() -> str:
+    d = os.environ.get('FLEX_RNN_CACHE')
+    if d:
+        return d
+    d = os.path.join(_HERE, '_kcache')
+    try:
+        os.makedirs(d, exist_ok=True)
+        if os.access(d, os.W_OK):
+            return d
+    except OSError:
+        pass
+    return os.path.join(os.path.expanduser('~'), '.cache', 'flex_rnn_amd')
+
+
+def source_key(name: str, src: str, opts: str = EMITTER_OPTS) -> str:
+    h = hashlib.sha256()
+    h.update(ARCH.encode())
+    h.update(b'\0')
+    h.update(opts.encode())
+    h.update(b'\0')
+    h.update(src.encode())
+    return f'{name}_{h.hexdigest()[:24]}'
+
+
+def compile_kernel(name: str, src: str, opts: str = EMITTER_OPTS, force: bool = False) -> str:
+    """Returns the path of the gfx950 code object for `src`, compiling on a cache miss
+    (or always, with `force`)."""
+    key = source_key(name, src, opts)
+    if force:
+        try:
+            os.remove(os.path.join(cache_dir(), key + '.hsaco'))
+        except FileNotFoundError:
+            pass
+    out = ctypes.create_string_buffer(4096)
+    b = src.encode()
+    rc = lib().frnn_compile(b, len(b), ARCH.encode(), opts.encode(), cache_dir().encode(), key.encode(), out, 4096)
+    _check(rc, f'compiling kernel {name}')
+    return out.value.decode()
+
+
+class Kernel:
+    def __init__(self, module: 'Module', name: str):
+        self.module = module
+        self.name = name
+        h = ctypes.c_void_p()
+        _check(lib().frnn_get_kernel(module.handle, name.encode(), ctypes.byref(h)), f'looking up kernel {name}')
+        self.handle = h
+
+    def launch(self, grid: Sequence[int], block: Sequence[int], args: bytes, stream: int = 0, lds_bytes: int = 0):
+        g = (ctypes.c_uint32 * 3)(*grid)
+        b = (ctypes.c_uint32 * 3)(*block)
+        buf = ctypes.create_string_buffer(args, len(args))
+        _check(lib().frnn_launch(self.handle, g, b, lds_bytes, ctypes.c_void_p(stream), buf, len(args)),
+               f'launching kernel {self.name}')
+
+
+class Module:
+    def __init__(self, path: str):
+        self.path = path
+        h = ctypes.c_void_p()
+        _check(lib().frnn_module_load(path.encode(), ctypes.byref(h)), f'loading code object {path}')
+        self.handle = h
+
+    def kernel(self, name: str) -> Kernel:
+        return Kernel(self, name)
+
+    def close(self):
+        if self.handle:
+            lib().frnn_module_free(self.handle)
+            self.handle = None
+
+
+def device_cus() -> int:
+    return lib().frnn_device_cus()
