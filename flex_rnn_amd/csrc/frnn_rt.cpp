@@ -269,6 +269,10 @@ int frnn_launch(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3]
   if (grid[1] > 65535 || grid[2] > 65535) return fail(FRNN_ERR_ARG, "frnn_launch: grid y/z larger than 65535");
   HipApi& h = hip();
   if (!h.ok) return fail(FRNN_ERR_NO_HIP, "%s", h.why.c_str());
+  // The block must be exactly as large as the kernel's explicit kernarg segment; kernels of
+  // this project take 8-byte fields only, so anything else is a packing mistake (a short block
+  // leaves the kernel reading arguments that were never set).
+  if (arg_bytes % 8 != 0) return fail(FRNN_ERR_ARG, "frnn_launch: argument block must be a whole number of 8-byte words");
   size_t sz = arg_bytes;
   void* extra[] = {(void*)0x01 /*BUFFER_POINTER*/, const_cast<void*>(args), (void*)0x02 /*BUFFER_SIZE*/, &sz,
                    (void*)0x03 /*END*/};

@@ -203,7 +203,7 @@ class _Args:
         return f'A.t[{self.slot(name)}].s[{d}]'
 
     def struct(self) -> str:
-        return f'struct Args {{ TArg t[{max(len(self.names), 1)}]; int B, T, H, M, nch; }};\n'
+        return f'struct Args {{ TArg t[{max(len(self.names), 1)}]; i64 B, T, H, M, nch; }};\n'
 
 
 def _col_expr(C: int, L: int) -> str:
@@ -255,7 +255,7 @@ class Emitter:
   const int mt = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int rloc = (wave * {G} + grp) * {R};
   const int row0 = mt * {MT} + rloc;
-  const int T = A.T, H = A.H, M = A.M, nch = A.nch;
+  const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T; (void)H; (void)nch;
 #define COL(c) {_col_expr(C, L)}
 #define ROWC(r) (min(row0 + (r), M - 1))
@@ -655,7 +655,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         b.append(f'''  const int tid = threadIdx.x;
   const int n = tid % {N};
   const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
-  const int T = A.T, H = A.H, M = A.M, nch = A.nch;
+  const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T;
   int ch = blockIdx.x * {IPB} + inst;
   const bool valid = ch < nch;

@@ -29,9 +29,17 @@ def kernel_specs(plan) -> List[KernelSpec]:
     return [em.fw(), em.bw1(), em.bw2()]
 
 
-def compile_plan(plan, force: bool = False) -> List[Tuple[KernelSpec, str]]:
-    """Emit + compile (or fetch from the cache) the three kernels.  Needs no GPU."""
-    return [(s, runtime.compile_kernel(s.name, s.source, force=force)) for s in kernel_specs(plan)]
+def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
+    """Emit + compile (or fetch from the cache) the three kernels.  Needs no GPU.  With
+    `force` a cached code object is rebuilt, once per key recorded in `seen`."""
+    out = []
+    for s in kernel_specs(plan):
+        key = runtime.source_key(s.name, s.source)
+        again = force and (seen is None or key not in seen)
+        if seen is not None:
+            seen.add(key)
+        out.append((s, runtime.compile_kernel(s.name, s.source, force=again)))
+    return out
 
 
 class CompiledPlan:
@@ -61,7 +69,7 @@ class CompiledPlan:
             buf += struct.pack('<q5q', t.data_ptr(), *_strides5(t))
         if not spec.tensors:
             buf += struct.pack('<q5q', 0, 0, 0, 0, 0, 0)
-        buf += struct.pack('<5i', pl.B, pl.T, pl.H, pl.M, pl.nchunks)
+        buf += struct.pack('<5q', pl.B, pl.T, pl.H, pl.M, pl.nchunks)
         env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
         grid = tuple(int(eval(g, {}, env)) for g in spec.grid)
         with th.cuda.device(dev):

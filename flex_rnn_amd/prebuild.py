@@ -61,10 +61,10 @@ def _is_full(name: str, i: int, j: int) -> bool:
 
 def warm(cases: Iterable = CASES, verbose: bool = False, force: bool = False) -> int:
     n = 0
-    done = set()
+    seen = set()
     for name, dims, dtype in cases:
         plan = plan_for(name, dims, dtype)
-        for spec, path in compile_plan(plan, force=force and (name, dims, dtype) not in done):
+        for spec, path in compile_plan(plan, force=force, seen=seen):
             n += 1
             if verbose:
                 print(f'  {name} {dims or "full"} {spec.name}: {path}')

@@ -63,8 +63,10 @@ int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out);
 
 /* Launch `k` with the given grid (in workgroups) and block (in threads) on `stream`
  * (a hipStream_t; NULL = default stream).  `args` points to `arg_bytes` bytes laid out
- * exactly as the kernel's parameter list (one by-value struct in this project).  Returns
- * after enqueueing; stream-ordered, never synchronises.
+ * exactly as the kernel's parameter list (one by-value struct of 8-byte fields in this
+ * project).  `arg_bytes` must equal the size of that parameter list and be a multiple of 8;
+ * a shorter block would leave the kernel with unset arguments.  Returns after enqueueing;
+ * stream-ordered, never synchronises.
  * Replaces: the generated `k<<<dim3(grid),dim3(threads)>>>(...)` launcher (to_cuda.py:245-247),
  * adding the stream and the error check the reference lacks. */
 int frnn_launch(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3],
