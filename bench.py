@@ -1,0 +1,144 @@
+#!/usr/bin/env python3
+"""Benchmark of the compiled recurrence on one MI355X.
+
+A step is one forward + backward pass of the headline workload (RWKV-7, B=8 T=1024 H=32,
+128x128 state, bf16 I/O) over one batch of synthetic inputs that already sit in HBM.  Prints
+one JSON line: whole-job tokens/s, the roofline figures of the dominant kernel (measured with
+events on the launch stream inside the timed region), and the CPU oracle timed on the host
+cores on a bounded sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_TFLOPS = 157.3      # MI355X vector fp32 peak (256 CU x 4 SIMD x 16 lanes x 4 flop x 2.4 GHz)
+PEAK_HBM_GBS = 8000.0
+
+# Algorithmic work per state element per timestep (full-tile arithmetic nodes of the traced
+# joint graph, a fused multiply-add counted as two; recomputation excluded) and algorithmic
+# HBM bytes per token, per workload: (fwd flop, bwd flop, gradient-kernel flop, fwd bytes, fwd+bwd bytes)
+WORK = {
+    'rwkv7': dict(flop_fwd=9, flop_bwd=19, flop_bw2=10, bytes_fwd=57344, bytes_all=163840),
+    'gated_delta_rule': dict(flop_fwd=7, flop_bwd=18, flop_bw2=9, bytes_fwd=32896, bytes_all=90496),
+    'mamba2': dict(flop_fwd=5, flop_bwd=18, flop_bw2=10, bytes_fwd=17024, bytes_all=42880),
+    'mamba1': dict(flop_fwd=8, flop_bwd=17, flop_bw2=8, bytes_fwd=49280, bytes_all=131456),
+}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--workload', default='rwkv7', choices=sorted(WORK))
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this build measures one GPU; --gpus {args.gpus} is not supported '
+              '(the recurrence shards over batch x head with no exchange, see DESIGN.md).', file=sys.stderr)
+        sys.exit(2)
+
+    import torch as th
+    import flex_rnn_amd
+    from flex_rnn_amd import configs
+
+    assert th.cuda.is_available(), 'bench.py needs a GPU'
+    dev = th.device('cuda:0')
+    name = args.workload
+    wl = configs.make(name, device='cpu')
+    B, T, H, M, N = wl.dims
+    dy, dS = configs.upstream_grads(wl)
+    f = flex_rnn_amd.jit(wl.step)
+    xs = [x.to(dev).requires_grad_() for x in wl.inputs]
+    ss = [s.to(dev).requires_grad_() for s in wl.states]
+    gy = None
+
+    def step():
+        nonlocal gy
+        res = f(*xs, *ss)
+        if gy is None:
+            gy = [g.to(dev).to(r.dtype) for g, r in zip(dy + dS, res)]
+        return th.autograd.grad(res, xs + ss, grad_outputs=gy)
+
+    for _ in range(max(args.warmup, 1)):
+        step()
+    th.cuda.synchronize()
+    compiled = f.forward_func.compiled
+    compiled.profile_events = []
+    th.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    th.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev = compiled.profile_events
+    compiled.profile_events = None
+    ms_per_step = wall * 1e3 / args.steps
+    tokens = B * T
+    value = tokens / (wall / args.steps)
+
+    per = {}
+    for kname, e0, e1 in ev:
+        per.setdefault(kname, []).append(e0.elapsed_time(e1))
+    kavg = {k: sum(v) / len(v) for k, v in per.items()}
+    dominant = max(kavg, key=kavg.get)
+    w = WORK[name]
+    elems = B * T * H * M * N
+    kflop = {'frnn_fw': w['flop_fwd'], 'frnn_bw1': w['flop_bwd'] - w['flop_bw2'], 'frnn_bw2': w['flop_bw2']}
+    achieved = kflop[dominant] * elems / (kavg[dominant] * 1e-3) / 1e12
+    gpu_ms = sum(kavg.values())
+    step_tflops = (w['flop_fwd'] + w['flop_bwd']) * elems / (gpu_ms * 1e-3) / 1e12
+    roofline = {
+        'bound': 'valu', 'kernel': dominant, 'achieved': round(achieved, 3), 'peak': PEAK_FP32_TFLOPS,
+        'unit': 'TFLOP/s', 'frac': round(achieved / PEAK_FP32_TFLOPS, 4), 'traffic': None,
+        'kernel_ms': {k: round(v, 4) for k, v in kavg.items()},
+        'step_achieved': round(step_tflops, 3), 'step_frac': round(step_tflops / PEAK_FP32_TFLOPS, 4),
+        'hbm_GBps_algorithmic': round(w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9, 1),
+        'hbm_frac': round(w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+    }
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(name)
+
+    out = {
+        'metric': 'fwd+bwd tokens/sec', 'value': round(value, 1), 'unit': 'tokens/s', 'n_gpus': 1,
+        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
+        'io_dtype': str(wl.dtype).replace('torch.', ''), 'data': 'synthetic',
+        'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
+        'roofline': roofline, 'cpu_baseline': cpu,
+        'gpu_kernel_ms_per_step': round(gpu_ms, 4),
+    }
+    print(json.dumps(out))
+
+
+def cpu_baseline(name, T_cpu=64):
+    """The CPU oracle (per-timestep loop + autograd) on the host cores, full B, H, M, N and a
+    short sequence (its cost is linear in T)."""
+    import torch as th
+    from flex_rnn_amd import configs
+    from oracle import recurrence
+    B, _, H, M, N = configs.DEFAULT_DIMS[name]
+    wl = configs.make(name, dims=(B, T_cpu, H, M, N))
+    dy, dS = configs.upstream_grads(wl)
+    xs = [x.float() for x in wl.inputs]
+    ss = [s.float() for s in wl.states]
+    times = []
+    for i in range(3):
+        t0 = time.perf_counter()
+        recurrence.loop_with_grads(wl.step, xs, ss, dy, dS, dtype=th.float32)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times[1:])[len(times[1:]) // 2] if len(times) > 1 else times[0]
+    return {'value': round(B * T_cpu / t, 1), 'unit': 'tokens/s', 'cores': th.get_num_threads(), 'kind': 'port',
+            'sample': f'{name} B{B} T{T_cpu} H{H} M{M} N{N} fp32, fwd+bwd through torch autograd, median of 2 after 1 warm-up',
+            'host_cpus': os.cpu_count()}
+
+
+if __name__ == '__main__':
+    main()

@@ -47,6 +47,8 @@ class CompiledPlan:
         self.plan = plan
         # (shape, stride, dtype) of the initial states: gradients w.r.t. them are laid out alike
         self.state_meta = state_meta
+        # when set to a list, every launch appends (kernel name, start event, end event)
+        self.profile_events = None
         built = compile_plan(plan)
         self.kernels = {}
         self.modules = []
@@ -74,7 +76,14 @@ class CompiledPlan:
         grid = tuple(int(eval(g, {}, env)) for g in spec.grid)
         with th.cuda.device(dev):
             stream = th.cuda.current_stream(dev).cuda_stream
-            kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
+            if self.profile_events is not None:
+                e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
+                e0.record()
+                kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
+                e1.record()
+                self.profile_events.append((kname, e0, e1))
+            else:
+                kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
 
     # ------------------------------------------------------------------ forward
     def forward(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):

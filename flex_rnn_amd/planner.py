@@ -255,4 +255,5 @@ def build_twopass(step: Callable, inputs, state, dryrun: bool = False, tile: Opt
         verify_meta(aux_, fw_out_meta[nout + 2 * nst:])
         return compiled.backward(doutput, dstateT_, tuple(inputs_), tuple(state_store_), aux_[0])
 
+    forward.compiled = backward.compiled = compiled
     return forward, backward, forward_meta, backward_meta
