@@ -15,7 +15,6 @@ aliasing `_to_copy`).
 """
 from __future__ import annotations
 
-import contextlib
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -38,29 +37,41 @@ def flat_step(step: Callable) -> Callable:
     return flat
 
 
-@contextlib.contextmanager
-def _isolated_tracing():
-    """Run a nested trace while an outer tracer (Dynamo / AOT-autograd fake mode)
-    is active: leave the outer fake mode and proxy modes for the duration.  The
-    reference needs a subprocess for this (trace_isolated.py:3-14)."""
-    from torch._subclasses.fake_tensor import unset_fake_temporarily
-    from torch.fx.experimental.proxy_tensor import disable_proxy_modes_tracing
-    with unset_fake_temporarily(), disable_proxy_modes_tracing():
-        with torch._C._DisableTorchDispatch() if False else contextlib.nullcontext():
-            yield
+def _needs_isolation() -> bool:
+    """True when the calling thread is inside another tracer (fake-tensor mode, proxy
+    tracing, functorch transform or a dispatcher callback with keys masked out)."""
+    if torch._guards.detect_fake_mode() is not None:
+        return True
+    if torch.utils._python_dispatch._get_current_dispatch_mode_stack():
+        return True
+    excl = str(torch._C._dispatch_tls_local_exclude_set())
+    return 'Functionalize' in excl or 'FuncTorchDynamicLayer' in excl
+
+
+def _run_isolated(fn):
+    """Dispatch-mode stacks, functorch layers and the dispatcher's include/exclude key sets are
+    all thread-local, so a nested trace started from inside another tracer (torch.compile
+    calling the op's fake implementation) runs on a fresh thread with default state.  The
+    reference pickles the graph through a subprocess for the same purpose
+    (/root/reference/flex_rnn/trace_isolated.py:3-14)."""
+    import concurrent.futures
+    with concurrent.futures.ThreadPoolExecutor(max_workers=1) as pool:
+        return pool.submit(fn).result()
 
 
 def trace_joint_fx(step: Callable, metas: Sequence[torch.Tensor]) -> Tuple[torch.fx.GraphModule, int]:
-    """`metas`: meta tensors [m,n] for inputs then states.  Returns the FX graph of
-    the joint function and the number of forward results (outputs + states)."""
+    """`metas`: tensors [m,n] (only shape and dtype are used) for inputs then states.  Returns
+    the FX graph of the joint function and the number of forward results (outputs + states)."""
     import torch._decomp
     from torch.fx.experimental.proxy_tensor import make_fx
 
     flat = flat_step(step)
     nargs = len(metas)
-    with _isolated_tracing():
-        metas = tuple(torch.empty(m.shape, dtype=m.dtype, device='meta') for m in metas)
-        outs = flat(*metas)
+    sig = [(tuple(m.shape), m.dtype) for m in metas]
+
+    def run():
+        args = tuple(torch.empty(s, dtype=d, device='meta') for s, d in sig)
+        outs = flat(*args)
 
         def fwbw(*a):
             x, dy = a[:nargs], a[nargs:]
@@ -70,8 +81,10 @@ def trace_joint_fx(step: Callable, metas: Sequence[torch.Tensor]) -> Tuple[torch
         cot = tuple(torch.empty(o.shape, dtype=o.dtype, device='meta') for o in outs)
         gm = make_fx(torch.func.functionalize(fwbw),
                      decomposition_table=torch._decomp.core_aten_decompositions(),
-                     tracing_mode='real')(*metas, *cot)
-    return gm, len(outs)
+                     tracing_mode='real')(*args, *cot)
+        return gm, len(outs)
+
+    return _run_isolated(run) if _needs_isolation() else run()
 
 
 # --------------------------------------------------------------------------- FX -> IR

@@ -1,0 +1,55 @@
+"""Runs one recurrence through the emitted kernels on the CPU (hipsim) and compares with the
+oracle.  Executed as a subprocess by tests/test_emit_sim.py so that a guard-page hit (SIGSEGV)
+fails one test instead of the whole session.
+
+usage: run_case.py <case> B,T,H,M,N <f32|bf16|f16> <against_end 0|1> [tol]
+"""
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+import torch as th
+
+import cases
+from flex_rnn_amd import configs, planner
+from hipsim import SimPlan
+from oracle import recurrence
+
+
+def main():
+    name, dims, dt, end = sys.argv[1], tuple(int(v) for v in sys.argv[2].split(',')), sys.argv[3], int(sys.argv[4])
+    dtype = {'f32': th.float32, 'bf16': th.bfloat16, 'f16': th.float16, 'f64': th.float64}[dt]
+    tol = float(sys.argv[5]) if len(sys.argv) > 5 else {'f32': 2e-5, 'f64': 2e-5, 'bf16': 1e-2, 'f16': 3e-3}[dt]
+    if name.startswith('cfg:'):
+        wl = configs.make(name[4:], dims=dims, dtype=dtype)
+        step, xs, ss = wl.step, wl.inputs, wl.states
+    else:
+        step, xs, ss = cases.make_inputs(name, *dims, dtype=dtype)
+    plan, fm, bm = planner.make_plan(step, xs, ss)
+    nout, nst = plan.part.noutputs, plan.part.nstates
+    sp = SimPlan(plan, state_meta=fm[nout:nout + nst], against_end=bool(end))
+    res = sp.forward(tuple(xs), tuple(ss))
+    outs, stT, sck, aux = res[:nout], res[nout:nout + nst], res[nout + nst:nout + 2 * nst], res[-1]
+    g = th.Generator().manual_seed(11)
+    dy = [th.randn(o.shape, generator=g) for o in outs]
+    dS = [th.randn(s.shape, generator=g) for s in ss]
+    dins, dst0 = sp.backward(tuple(d.to(o.dtype) for d, o in zip(dy, outs)),
+                             tuple(d.to(s.dtype) for d, s in zip(dS, stT)), tuple(xs), sck, aux)
+    dyq = [d.to(o.dtype) for d, o in zip(dy, outs)]
+    dSq = [d.to(s.dtype) for d, s in zip(dS, stT)]
+    want = recurrence.loop_with_grads(step, xs, ss, dyq, dSq)
+    got = list(outs) + list(stT) + list(dins) + list(dst0)
+    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    worst = 0.0
+    for a, b in zip(got, want):
+        assert a.shape == b.shape, (a.shape, b.shape)
+        worst = max(worst, recurrence.rel_err(a, b))
+    print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e}')
+    assert worst < tol, worst
+
+
+if __name__ == '__main__':
+    main()

@@ -1,0 +1,141 @@
+"""Decorator surface, operand validation, dry-run metadata and fake-tensor behaviour - the
+parts of the boundary that need no GPU."""
+import pytest
+import torch as th
+
+import flex_rnn_amd
+from flex_rnn_amd import ops, planner
+from flex_rnn_amd.planner import split_list, verify_meta
+
+import cases
+
+
+def test_arity_inference_and_surface():
+    f = flex_rnn_amd.jit(ops.rwkv7)
+    assert (f.ninputs, f.nstates, f.noutputs) == (6, 1, 1)
+    g = flex_rnn_amd.jit(ops.rwkv4)
+    assert (g.ninputs, g.nstates, g.noutputs) == (4, 3, 1)
+    h = flex_rnn_amd.jit(ops.mlstm_gates)
+    assert (h.ninputs, h.nstates, h.noutputs) == (2, 1, 3)
+    for attr in ('step', 'apply', 'forward_func', 'backward_func', 'naive', 'naive_fp64', 'build_call'):
+        assert hasattr(f, attr)
+    assert f.forward_func is None and f.backward_func is None        # nothing compiled yet
+    assert flex_rnn_amd.__version__ == '0.2'
+    assert callable(flex_rnn_amd.check_grad) and callable(flex_rnn_amd.benchmark)
+    # explicit arity for a step with *args
+    k = flex_rnn_amd.jit(lambda *a: ops.gla(*a), n_step_args=5)
+    assert (k.ninputs, k.nstates) == (4, 1)
+
+
+def test_apply_is_reassignable():
+    f = flex_rnn_amd.jit(ops.gla)
+    step, xs, ss = cases.make_inputs('gla', 1, 4, 1, 4, 4, dtype=th.float32)
+    f.apply = f.naive_fp64
+    y, S = f(*xs, *ss)
+    assert y.dtype == th.float64 and y.shape == (1, 4, 1, 4)
+
+
+def test_split_list_and_verify_meta():
+    assert split_list([1, 2, 3, 4], [1, 3]) == [[1], [2, 3, 4]]
+    with pytest.raises(AssertionError):
+        split_list([1, 2, 3], [1, 1])
+    a = th.empty(2, 1, 4)
+    verify_meta([a], [th.empty(2, 1, 4).as_strided((2, 1, 4), (4, 99, 1))])     # stride of a size-1 dim is ignored
+    with pytest.raises(AssertionError, match='shape'):
+        verify_meta([a], [th.empty(2, 2, 4)])
+    with pytest.raises(AssertionError, match='stride'):
+        verify_meta([a], [th.empty(4, 1, 2).permute(2, 1, 0)])
+    with pytest.raises(AssertionError, match='dtype'):
+        verify_meta([a], [th.empty(2, 1, 4, dtype=th.bfloat16)])
+
+
+def test_operand_validation_messages():
+    S = th.zeros(2, 3, 4, 8)
+    q = th.zeros(2, 5, 3, 1, 8)
+    with pytest.raises(AssertionError, match='invalid shape'):
+        planner.classify([th.zeros(2, 5, 3, 8)], [S])
+    with pytest.raises(AssertionError, match='incompatible'):
+        planner.classify([q, th.zeros(2, 5, 2, 4, 1)], [S])
+    with pytest.raises(AssertionError, match='both a matrix'):
+        planner.classify([q, th.zeros(2, 5, 3, 4, 8)], [S])
+    with pytest.raises(AssertionError, match='!='):
+        planner.classify([q], [th.zeros(2, 1, 4, 8)])
+    with pytest.raises(AssertionError, match='dtype'):
+        planner.classify([q.to(th.int32)], [S])
+    dims, cls, bc = planner.classify([q, th.zeros(2, 5, 3, 4, 1), th.zeros(1, 1, 3, 1, 1), th.zeros(1, 1, 3, 4, 8)], [S])
+    assert dims == [2, 5, 3, 4, 8] and cls == ['row', 'col', 'scalar', 'mat']
+    assert bc == [(False, False, False), (False, False, False), (True, True, False), (True, True, False)]
+
+
+def test_dryrun_metadata():
+    step, xs, ss = cases.make_inputs('rwkv7', 2, 32, 3, 16, 32, dtype=th.bfloat16)
+    ss = [s.float().mT.contiguous().mT for s in ss]                 # transposed-stride state
+    fw_meta, bw_meta = planner.build_twopass(step, xs, ss, dryrun=True)
+    (ysh, yst, ydt), (ssh, sst, sdt), (cksh, _, ckdt), (ash, _, adt) = fw_meta
+    assert tuple(ysh) == (2, 32, 3, 16) and ydt == th.bfloat16           # step ends in .to(r.dtype)
+    assert tuple(ssh) == (2, 3, 16, 32) and tuple(sst) == tuple(ss[0].stride()) and sdt == th.float32
+    assert tuple(cksh) == (2, 3, 2, 16, 32) and ckdt == th.float32       # a checkpoint every 16 steps
+    assert tuple(ash) == (1, 2, 3, 32, 16) and adt == th.float32         # one saved row sum per step
+    assert len(bw_meta) == 7
+    for (sh, st, dt), x in zip(bw_meta, xs + ss):
+        assert tuple(sh) == tuple(x.shape) and dt == x.dtype
+
+
+def test_fake_tensor_mode_uses_dry_run():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    f = flex_rnn_amd.jit(ops.delta_rule)
+    step, xs, ss = cases.make_inputs('delta_rule', 2, 16, 2, 8, 8, dtype=th.float32)
+    with FakeTensorMode() as mode:
+        fx = [mode.from_tensor(x) for x in xs]
+        fs = [mode.from_tensor(s) for s in ss]
+        y, S = f(*fx, *fs)
+    assert tuple(y.shape) == (2, 16, 2, 8) and tuple(S.shape) == (2, 2, 8, 8)
+    assert f.forward_func is None            # nothing was compiled or launched
+    assert hasattr(f, 'fw_meta') and hasattr(f, 'bw_meta')
+
+
+def test_compiled_path_has_no_cpu_fallback(runtime_lib):
+    if th.cuda.is_available():
+        pytest.skip('a GPU is present')
+    f = flex_rnn_amd.jit(ops.delta_rule)
+    step, xs, ss = cases.make_inputs('delta_rule', 1, 16, 1, 16, 16, dtype=th.float32)
+    with pytest.raises((RuntimeError, AssertionError)):
+        f(*xs, *ss)
+
+
+def test_unsupported_op_is_named():
+    def bad(x, S):
+        S = S + th.cumsum(x, -1)
+        return S.sum(-1, True), S
+    with pytest.raises(NotImplementedError, match='cumsum'):
+        planner.make_plan(bad, [th.zeros(1, 2, 1, 1, 4)], [th.zeros(1, 1, 4, 4)])
+
+
+def test_drop_in_alias_package():
+    import flex_rnn
+    assert flex_rnn.jit is flex_rnn_amd.jit and flex_rnn.check_grad is flex_rnn_amd.check_grad
+
+
+def test_dynamo_traces_through_the_op_without_graph_break(runtime_lib):
+    """torch.compile sees one opaque op: the captured graph holds a single flex_rnn::fw_* call
+    and no graph break occurs.  (Running it needs a GPU; only the capture is checked here.)"""
+    if th.cuda.is_available():
+        pytest.skip('covered by the GPU test')
+    f = flex_rnn_amd.jit(ops.delta_rule)
+    step, xs, ss = cases.make_inputs('delta_rule', 1, 16, 2, 8, 8, dtype=th.float32)
+    graphs = []
+
+    def backend(gm, example_inputs):
+        graphs.append(gm)
+        return gm.forward
+
+    def layer(q, k, v, beta, S):
+        y, S = f(q * 2, k, v, beta, S)
+        return y + 1, S
+
+    compiled = th.compile(layer, backend=backend, fullgraph=True)
+    with pytest.raises((RuntimeError, AssertionError)):      # no GPU: the real kernel cannot run
+        compiled(*xs, *ss)
+    assert len(graphs) == 1
+    targets = [str(n.target) for n in graphs[0].graph.nodes if n.op == 'call_function']
+    assert sum('flex_rnn.fw_' in t for t in targets) == 1, targets

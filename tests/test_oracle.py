@@ -1,0 +1,162 @@
+"""Pins the CPU oracle (oracle/recurrence.py) with closed forms, brute force and invariants,
+and checks the package's `jit.naive` against it."""
+import math
+
+import pytest
+import torch as th
+
+import flex_rnn_amd
+from flex_rnn_amd import ops
+from oracle import recurrence
+
+D = th.float64
+
+
+def rnd(*shape, seed=0):
+    return th.randn(*shape, generator=th.Generator().manual_seed(seed), dtype=D)
+
+
+def test_decay_linear_attention_closed_form():
+    # S_t = S_{t-1} * w_t + v_t k_t^T ;  y_t = S_t q_t
+    B, T, H, M, N = 2, 9, 3, 4, 5
+    q, k = rnd(B, T, H, 1, N, seed=1), rnd(B, T, H, 1, N, seed=2)
+    v = rnd(B, T, H, M, 1, seed=3)
+    w = th.sigmoid(rnd(B, T, H, 1, N, seed=4))
+    S0 = rnd(B, H, M, N, seed=5)
+
+    def step(q, k, v, w, S):
+        S = S * w + v * k
+        return (S * q).sum(-1, True), S
+
+    (y,), (ST,) = recurrence.run_loop(step, [q, k, v, w], [S0])
+    # closed form with explicit products (no shared code path with the loop)
+    logw = th.log(w[:, :, :, 0])                       # [B,T,H,N]
+    cum = th.cumsum(logw, dim=1)                       # prod_{r<=t} w_r
+    y_ref = th.zeros(B, T, H, M, dtype=D)
+    for t in range(T):
+        acc = (S0 * th.exp(cum[:, t])[:, :, None, :] * q[:, t]).sum(-1)        # initial-state term
+        for s in range(t + 1):
+            decay = th.exp(cum[:, t] - cum[:, s])                              # prod_{s<r<=t} w_r
+            dot = (q[:, t, :, 0] * k[:, s, :, 0] * decay).sum(-1)              # [B,H]
+            acc = acc + v[:, s, :, :, 0] * dot[:, :, None]
+        y_ref[:, t] = acc
+    assert recurrence.rel_err(y, y_ref) < 1e-12
+    ST_ref = S0 * th.exp(cum[:, -1])[:, :, None, :]
+    for s in range(T):
+        ST_ref = ST_ref + v[:, s] * (k[:, s] * th.exp(cum[:, -1] - cum[:, s])[:, :, None, :])
+    assert recurrence.rel_err(ST, ST_ref) < 1e-12
+
+
+def test_vector_state_scan_closed_form():
+    # N = 1: s_t = exp(g_t) s_{t-1} + x_t
+    B, T, M = 2, 11, 6
+    x, g = rnd(B, T, 1, M, 1, seed=1), -th.sigmoid(rnd(B, T, 1, M, 1, seed=2))
+    s0 = rnd(B, 1, M, 1, seed=3)
+    (y,), (sT,) = recurrence.run_loop(ops.hgrn, [x, g], [s0])
+    G = th.cumsum(g[:, :, 0, :, 0], dim=1)               # [B,T,M]
+    ref = th.exp(G) * s0[:, 0, :, 0][:, None]
+    for s in range(T):
+        ref[:, s:] += th.exp(G[:, s:] - G[:, s:s + 1]) * x[:, s:s + 1, 0, :, 0]
+    assert recurrence.rel_err(y[:, :, 0], ref) < 1e-12
+    assert recurrence.rel_err(sT[:, 0, :, 0], ref[:, -1]) < 1e-12
+
+
+def test_single_step_delta_rule_matrix_form():
+    B, H, M, N = 2, 2, 3, 4
+    q, k = rnd(B, 1, H, 1, N, seed=1), rnd(B, 1, H, 1, N, seed=2)
+    v, beta = rnd(B, 1, H, M, 1, seed=3), th.sigmoid(rnd(B, 1, H, 1, 1, seed=4))
+    S0 = rnd(B, H, M, N, seed=5)
+    (y,), (S1,) = recurrence.run_loop(ops.delta_rule, [q, k, v, beta], [S0])
+    kk = k[:, 0, :, 0]                                                    # [B,H,N]
+    I = th.eye(N, dtype=D)
+    P = I - beta[:, 0, :, 0, 0][:, :, None, None] * kk[..., :, None] * kk[..., None, :]
+    ref = S0 @ P + beta[:, 0] * v[:, 0] * k[:, 0]
+    assert recurrence.rel_err(S1, ref) < 1e-12
+    assert recurrence.rel_err(y[:, 0], (ref @ q[:, 0, :, 0][..., None])[..., 0]) < 1e-12
+
+
+def test_mamba_constant_inputs_geometric_series():
+    B, T, H, M, N = 1, 13, 2, 3, 4
+    delta, xval = 0.3, 0.7
+    A = -th.arange(1, N + 1, dtype=D).view(1, 1, 1, 1, N).expand(1, 1, H, M, N).contiguous()
+    x = th.full((B, T, H, M, 1), xval, dtype=D)
+    dl = th.full((B, T, H, M, 1), delta, dtype=D)
+    Bm, Cm = th.ones(B, T, 1, 1, N, dtype=D), th.ones(B, T, 1, 1, N, dtype=D)
+    S0 = th.zeros(B, H, M, N, dtype=D)
+    (y,), (ST,) = recurrence.run_loop(ops.mamba, [x, dl, A, Bm, Cm], [S0])
+    r = th.exp(delta * A[0, 0])                                   # [H,M,N]
+    ST_ref = delta * xval * (1 - r ** T) / (1 - r)
+    assert recurrence.rel_err(ST[0], ST_ref) < 1e-12
+    t = 5
+    y_ref = (delta * xval * (1 - r ** (t + 1)) / (1 - r)).sum(-1)
+    assert recurrence.rel_err(y[0, t], y_ref) < 1e-12
+
+
+def _rwkv7_inputs(B, T, H, M, N, seed=0):
+    r, k = rnd(B, T, H, 1, N, seed=seed), rnd(B, T, H, 1, N, seed=seed + 1)
+    w = th.exp(-th.exp(rnd(B, T, H, 1, N, seed=seed + 2)))
+    kk = th.nn.functional.normalize(rnd(B, T, H, 1, N, seed=seed + 3), dim=-1)
+    a, b = -kk, kk * th.sigmoid(rnd(B, T, H, 1, N, seed=seed + 4))
+    v = rnd(B, T, H, M, 1, seed=seed + 5)
+    return [r, w, k, v, a, b], [rnd(B, H, M, N, seed=seed + 6)]
+
+
+def test_invariants_permutation_chunking_broadcast():
+    xs, ss = _rwkv7_inputs(3, 8, 2, 4, 4)
+    (y,), (ST,) = recurrence.run_loop(ops.rwkv7_decay, xs, ss)
+    perm = th.tensor([2, 0, 1])
+    (yp,), (STp,) = recurrence.run_loop(ops.rwkv7_decay, [x[perm] for x in xs], [s[perm] for s in ss])
+    assert th.equal(yp, y[perm]) and th.equal(STp, ST[perm])
+    # chunked call with state hand-off
+    (y1,), s1 = recurrence.run_loop(ops.rwkv7_decay, [x[:, :3] for x in xs], ss)
+    (y2,), s2 = recurrence.run_loop(ops.rwkv7_decay, [x[:, 3:] for x in xs], s1)
+    assert th.equal(th.cat([y1, y2], 1), y) and th.equal(s2[0], ST)
+    # broadcast input == materialised input
+    xb = list(xs)
+    xb[1] = xs[1][:, :1, :1]                                    # decay shared over time and heads
+    xm = list(xs)
+    xm[1] = xb[1].expand(-1, 8, 2, -1, -1).contiguous()
+    ob, om = recurrence.run_loop(ops.rwkv7_decay, xb, ss), recurrence.run_loop(ops.rwkv7_decay, xm, ss)
+    assert th.equal(ob[0][0], om[0][0])
+
+
+def test_gradients_against_finite_differences():
+    xs, ss = _rwkv7_inputs(1, 3, 1, 2, 2, seed=7)
+    dy, dS = rnd(1, 3, 1, 2, seed=20), rnd(1, 1, 2, 2, seed=21)
+    _, _, dins, dst = recurrence.loop_with_grads(ops.rwkv7_decay, xs, ss, [dy], [dS])
+
+    def loss(vals):
+        (y,), (ST,) = recurrence.run_loop(ops.rwkv7_decay, vals[:6], vals[6:])
+        return (y * dy).sum() + (ST * dS).sum()
+
+    vals = [x.clone() for x in xs + ss]
+    grads = dins + dst
+    eps = 1e-6
+    for i, g in enumerate(grads):
+        flat = vals[i].view(-1)
+        for j in range(0, flat.numel(), max(1, flat.numel() // 3)):
+            old = flat[j].item()
+            flat[j] = old + eps
+            lp = loss(vals)
+            flat[j] = old - eps
+            lm = loss(vals)
+            flat[j] = old
+            fd = (lp - lm) / (2 * eps)
+            assert abs(fd - g.reshape(-1)[j]) < 1e-6 * max(1.0, abs(fd)), (i, j, fd, g.reshape(-1)[j])
+
+
+@pytest.mark.parametrize('dtype', [th.float32, th.bfloat16])
+def test_package_naive_matches_oracle(dtype):
+    xs, ss = _rwkv7_inputs(2, 6, 2, 4, 8)
+    xs = [x.to(dtype) for x in xs]
+    ss = [s.to(th.float32).mT.contiguous().mT for s in ss]         # non-contiguous state layout
+    f = flex_rnn_amd.jit(ops.rwkv7_decay)
+    y, ST = f.naive(*xs, *ss)
+    (yo,), (STo,) = recurrence.run_loop(ops.rwkv7_decay, xs, ss, dtype=th.float32)
+    assert y.dtype == yo.dtype == th.float32          # outputs come back in the loop dtype
+    assert ST.dtype == ss[0].dtype and ST.stride() == ss[0].stride()
+    assert recurrence.rel_err(y, yo) == 0 and recurrence.rel_err(ST, STo) == 0
+    y64, _ = f.naive_fp64(*xs, *ss)
+    assert y64.dtype == th.float64
+    (y64o,), _ = recurrence.run_loop(ops.rwkv7_decay, xs, ss, dtype=th.float64)
+    assert recurrence.rel_err(y64, y64o) == 0

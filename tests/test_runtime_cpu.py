@@ -1,0 +1,95 @@
+"""CPU tests of the C-ABI runtime: exported symbols, compile cache, error reporting, and the
+launch marshalling (against a stand-in HIP runtime)."""
+import ctypes
+import os
+import re
+import subprocess
+import sys
+import textwrap
+
+import pytest
+
+from flex_rnn_amd import runtime
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TRIVIAL = '#include <hip/hip_runtime.h>\nextern "C" __global__ void k(float* p) { p[threadIdx.x] = 1.0f; }\n'
+
+
+def test_library_exports_every_declared_symbol(runtime_lib):
+    hdr = open(os.path.join(ROOT, 'include', 'frnn_rt.h')).read()
+    declared = set(re.findall(r'\b(frnn_\w+)\s*\(', hdr))
+    declared -= {'frnn_module_s'}
+    assert declared == set(runtime.EXPORTS)
+    for name in declared:
+        assert hasattr(runtime_lib, name), name
+    assert runtime_lib.frnn_version() >= 100
+
+
+def test_compile_cache_hit_and_miss(runtime_lib, tmp_path, monkeypatch):
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    p1 = runtime.compile_kernel('k', TRIVIAL)
+    assert os.path.getsize(p1) > 0 and p1.startswith(str(tmp_path)) and p1.endswith('.hsaco')
+    assert os.path.isfile(p1[:-6] + '.hip')
+    m1 = os.path.getmtime(p1)
+    assert runtime.compile_kernel('k', TRIVIAL) == p1 and os.path.getmtime(p1) == m1     # hit
+    p2 = runtime.compile_kernel('k', TRIVIAL + '// other\n')
+    assert p2 != p1                                                                       # key = source hash
+    # a truncated cache entry is rebuilt when asked to
+    runtime.compile_kernel('k', TRIVIAL, force=True)
+    assert os.path.getsize(p1) > 0
+
+
+def test_compile_error_is_reported(runtime_lib, tmp_path, monkeypatch):
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    with pytest.raises(RuntimeError, match='hipcc failed'):
+        runtime.compile_kernel('bad', 'this is not HIP\n')
+    assert not [f for f in os.listdir(tmp_path) if f.endswith('.hsaco')]
+
+
+def test_bad_key_and_null_arguments(runtime_lib, tmp_path):
+    out = ctypes.create_string_buffer(256)
+    rc = runtime_lib.frnn_compile(b'x', 1, b'gfx950', b'', str(tmp_path).encode(), b'../evil', out, 256)
+    assert rc == 1 and b'key' in runtime_lib.frnn_last_error()
+    rc = runtime_lib.frnn_compile(None, 0, b'gfx950', b'', str(tmp_path).encode(), b'k', out, 256)
+    assert rc == 1
+
+
+def test_load_without_gpu_fails_loudly(runtime_lib, tmp_path, monkeypatch):
+    import torch
+    if torch.cuda.is_available():
+        pytest.skip('a GPU is present')
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    path = runtime.compile_kernel('k', TRIVIAL)
+    with pytest.raises(RuntimeError):
+        runtime.Module(path)
+
+
+def test_launch_marshalling_against_stand_in_hip(runtime_lib, tmp_path):
+    so = tmp_path / 'libfakehip.so'
+    subprocess.run(['g++', '-shared', '-fPIC', '-o', str(so), os.path.join(ROOT, 'tests', 'fakehip', 'fakehip.cpp')], check=True)
+    code = textwrap.dedent(f'''
+        import ctypes, struct, sys
+        sys.path.insert(0, {ROOT!r})
+        fake = ctypes.CDLL({str(so)!r}, mode=ctypes.RTLD_GLOBAL)
+        from flex_rnn_amd import runtime
+        assert runtime.device_cus() == 256
+        m = runtime.Module('/nonexistent'); k = m.kernel('x')
+        buf = struct.pack('<q5q', 0x7f0012345678, 1, 2, 3, 4, 5) + struct.pack('<5q', 7, 8, 9, 10, 11)
+        k.launch((2, 3, 4), (64, 1, 1), buf, stream=0xabc)
+        n = ctypes.c_size_t.in_dll(fake, 'g_nargs').value
+        got = bytes((ctypes.c_ubyte * 8192).in_dll(fake, 'g_args'))[:n]
+        assert got == buf and ctypes.c_int.in_dll(fake, 'g_extra_ok').value == 1
+        assert list((ctypes.c_uint * 7).in_dll(fake, 'g_dims')) == [2, 3, 4, 64, 1, 1, 0]
+        assert ctypes.c_void_p.in_dll(fake, 'g_stream').value == 0xabc
+        for bad in [dict(args=buf[:-4]), dict(grid=(0, 1, 1)), dict(block=(2048, 1, 1)), dict(grid=(1, 70000, 1))]:
+            kw = dict(grid=(1, 1, 1), block=(64, 1, 1), args=buf); kw.update(bad)
+            try:
+                k.launch(kw['grid'], kw['block'], kw['args'])
+            except RuntimeError as e:
+                assert 'frnn_launch' in str(e), e
+            else:
+                raise SystemExit('accepted ' + str(bad))
+        print('ok')
+    ''')
+    r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
+    assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr
