@@ -63,6 +63,21 @@ template <> __device__ __forceinline__ float ldf<1>(const void* p, i64 i) {
 template <> __device__ __forceinline__ float ldf<2>(const void* p, i64 i) { return (float)((const _Float16*)p)[i]; }
 template <> __device__ __forceinline__ float ldf<3>(const void* p, i64 i) { return (float)((const double*)p)[i]; }
 
+// raw (unconverted) load into a 32-bit register and its conversion: lets a prefetch stay in flight
+// without an instruction that consumes the loaded value
+template <int DT> __device__ __forceinline__ unsigned ldr(const void* p, i64 i);
+template <> __device__ __forceinline__ unsigned ldr<0>(const void* p, i64 i) { return ((const unsigned*)p)[i]; }
+template <> __device__ __forceinline__ unsigned ldr<1>(const void* p, i64 i) { return ((const u16_t*)p)[i]; }
+template <> __device__ __forceinline__ unsigned ldr<2>(const void* p, i64 i) { return ((const u16_t*)p)[i]; }
+template <> __device__ __forceinline__ unsigned ldr<3>(const void* p, i64 i) {
+  return __builtin_bit_cast(unsigned, (float)((const double*)p)[i]);
+}
+template <int DT> __device__ __forceinline__ float cvr(unsigned u);
+template <> __device__ __forceinline__ float cvr<0>(unsigned u) { return __builtin_bit_cast(float, u); }
+template <> __device__ __forceinline__ float cvr<1>(unsigned u) { return __builtin_bit_cast(float, u << 16); }
+template <> __device__ __forceinline__ float cvr<2>(unsigned u) { return (float)__builtin_bit_cast(_Float16, (u16_t)u); }
+template <> __device__ __forceinline__ float cvr<3>(unsigned u) { return __builtin_bit_cast(float, u); }
+
 template <int DT> __device__ __forceinline__ void stf(void* p, i64 i, float v);
 template <> __device__ __forceinline__ void stf<0>(void* p, i64 i, float v) { ((float*)p)[i] = v; }
 template <> __device__ __forceinline__ void stf<1>(void* p, i64 i, float v) {
@@ -206,6 +221,47 @@ class _Args:
         return f'struct Args {{ TArg t[{max(len(self.names), 1)}]; i64 B, T, H, M, nch; }};\n'
 
 
+class _Stager:
+    """Global -> LDS staging of per-timestep operands for TS timesteps, split in two phases so
+    that the loads of the next chunk are in flight while the current one is computed:
+    `load(t0)` issues every load of the chunk back to back into registers (raw bits),
+    `write()` converts them to fp32 and stores them to LDS."""
+
+    def __init__(self, TS: int, NT: int):
+        self.TS, self.NT = TS, NT
+        self.items = []          # (lds name, row length, dtype code, pointer expr, index fn(t0, tt_, x_))
+
+    def add(self, name, ln, dt, ptr, idx_fn):
+        self.items.append((name, ln, dt, ptr, idx_fn))
+
+    def _iters(self, ln):
+        return (self.TS * ln + self.NT - 1) // self.NT
+
+    def decls(self) -> str:
+        out = ''
+        for name, ln, dt, ptr, fn in self.items:
+            out += f'  __shared__ float {name}[{self.TS}][{ln}];\n  unsigned pf_{name}[{self._iters(ln)}];\n'
+        return out
+
+    def _loop(self, ln, body, ind):
+        tot = self.TS * ln
+        guard = '' if tot % self.NT == 0 else f'if (e_ < {tot}) '
+        return (f'#pragma unroll\n{ind}for (int it_ = 0; it_ < {self._iters(ln)}; it_++) {{ const int e_ = tid + it_ * {self.NT}; '
+                f'const int tt_ = e_ / {ln}, x_ = e_ % {ln}; (void)tt_; (void)x_; {guard}{body} }}\n')
+
+    def load(self, t0: str, ind: str) -> str:
+        out = ''
+        for name, ln, dt, ptr, fn in self.items:
+            out += self._loop(ln, f'pf_{name}[it_] = ldr<{dt}>({ptr}, {fn(t0, "tt_", "x_")});', ind)
+        return out
+
+    def write(self, ind: str) -> str:
+        out = ''
+        for name, ln, dt, ptr, fn in self.items:
+            out += self._loop(ln, f'{name}[tt_][x_] = cvr<{dt}>(pf_{name}[it_]);', ind)
+        return out
+
+
 def _col_expr(C: int, L: int) -> str:
     """Column owned by (lane-in-group l, element c).  With C >= 4 a lane owns float4
     pieces, interleaved across the group so that 16 lanes x 16 B is one contiguous row
@@ -262,27 +318,17 @@ class Emitter:
 ''')
         return src, MT
 
-    def _stage_decl(self, nm: str, ext, TS: int, MT: int) -> str:
-        N = self.plan.N
-        ln = (N if ext[1] else 1) if not ext[0] else MT
-        return f'  __shared__ float {nm}[{TS}][{ln}];\n'
-
-    def _stage_in(self, A: _Args, i: int, TS: int, MT: int, NT: int, t0: str) -> str:
-        """Cooperative global -> LDS copy of input i for timesteps [t0, t0+TS)."""
+    def _stage_input(self, st: '_Stager', A: _Args, i: int, MT: int):
         ext = self.in_ext(i)
         N = self.plan.N
         dt = DT_CODE[self.plan.in_dtypes[i]]
         if ext == (False, True):
-            ln, idx = N, self._in_index(A, i, t=f'{t0} + tt_', n='x_')
-            guard = ''
+            st.add(f's_in{i}', N, dt, A.p(f'in{i}'), lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}', n=x))
         elif ext == (True, False):
-            ln, idx = MT, self._in_index(A, i, t=f'{t0} + tt_', m=f'min(mt * {MT} + x_, M - 1)')
-            guard = ''
+            st.add(f's_in{i}', MT, dt, A.p(f'in{i}'),
+                   lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}', m=f'min(mt * {MT} + {x}, M - 1)'))
         else:
-            ln, idx = 1, self._in_index(A, i, t=f'{t0} + tt_')
-            guard = ''
-        return (f'    for (int e_ = tid; e_ < {TS * ln}; e_ += {NT}) {{ int tt_ = e_ / {ln}, x_ = e_ % {ln}; (void)x_;\n'
-                f'      s_in{i}[tt_][x_] = ldf<{dt}>({A.p(f"in{i}")}, {idx}); }}\n')
+            st.add(f's_in{i}', 1, dt, A.p(f'in{i}'), lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}'))
 
     def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str) -> str:
         """Registers <- staged LDS operand for timestep tt."""
@@ -328,9 +374,11 @@ class Emitter:
         src, MT = self._row_kernel_common(A, used_in, R, W)
         body = []
         # staging buffers
+        stg = _Stager(TS, NT)
         for i in used_in:
             if self.tdep[i]:
-                body.append(self._stage_decl(f's_in{i}', self.in_ext(i), TS, MT))
+                self._stage_input(stg, A, i, MT)
+        body.append(stg.decls())
         for k in range(nout):
             body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
         for k in range(naux):
@@ -346,6 +394,7 @@ class Emitter:
         for i in used_in:
             if not self.tdep[i]:
                 body.append(self._load_const_input(A, i, R, C))
+        body.append(stg.load('0', '  '))
         body.append(f'  for (int t0 = 0; t0 < T; t0 += {TS}) {{\n')
         # checkpoint
         body.append(f'    if (t0 % {DT} == 0) {{\n')
@@ -355,10 +404,9 @@ class Emitter:
                         f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
                         f'((float*){A.p(f"sck{k}")})[{self._ck_index(f"t0 / {DT}")}] = S{k}[r][c]; }}\n')
         body.append('    }\n    __syncthreads();\n')
-        for i in used_in:
-            if self.tdep[i]:
-                body.append(self._stage_in(A, i, TS, MT, NT, 't0'))
+        body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
+        body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
         body.append(f'#pragma unroll 2\n    for (int tt = 0; tt < {TS}; tt++) {{\n')
         call = []
         for nm_ in used:
@@ -445,13 +493,19 @@ class Emitter:
         used_dout = [k for k in range(nout) if p.dout_names[k] in used_all]
         src, MT = self._row_kernel_common(A, used_in, R, W)
         body = []
+        stg = _Stager(TS, NT)
         for i in used_in:
             if self.tdep[i]:
-                body.append(self._stage_decl(f's_in{i}', self.in_ext(i), TS, MT))
+                self._stage_input(stg, A, i, MT)
         for k in used_aux:
-            body.append(f'  __shared__ float s_aux{k}[{TS}][{MT}];\n')
+            stg.add(f's_aux{k}', MT, 0, A.p('aux'),
+                    lambda t0, tt, x, k=k: f'((((i64){k} * A.B + b) * H + h) * T + ({t0} + {tt})) * M + min(mt * {MT} + {x}, M - 1)')
         for k in used_dout:
-            body.append(f'  __shared__ float s_dy{k}[{TS}][{MT}];\n')
+            nm = f'dout{k}'
+            stg.add(f's_dy{k}', MT, DT_CODE[plan.out_dtypes[k]], A.p(nm),
+                    lambda t0, tt, x, nm=nm: (f'(i64)b * {A.s(nm, 0)} + (i64)({t0} + {tt}) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + '
+                                               f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'))
+        body.append(stg.decls())
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
         for i in tdep_col:
@@ -471,6 +525,7 @@ class Emitter:
                 body.append(self._load_const_input(A, i, R, C))
         for i in const_col:
             body.append(f'  float gacc{i}[{rrs}][1];\n#pragma unroll\n  for (int r = 0; r < {rrs}; r++) gacc{i}[r][0] = 0.0f;\n')
+        body.append(stg.load(f'T - {TS}', '  '))
         body.append(f'  for (int t0 = T - {TS}; t0 >= 0; t0 -= {TS}) {{\n')
         body.append(f'    if ((t0 + {TS}) % {DT} == 0) {{\n')
         for k in range(nst):
@@ -479,21 +534,9 @@ class Emitter:
                         f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
                         f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"(t0 + {TS}) / {DT} - 1")}] = D{k}[r][c]; }}\n')
         body.append('    }\n    __syncthreads();\n')
-        for i in used_in:
-            if self.tdep[i]:
-                body.append(self._stage_in(A, i, TS, MT, NT, 't0'))
-        stage_rows = (f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; '
-                      f'int m_ = min(mt * {MT} + x_, M - 1);\n')
-        if used_aux or used_dout:
-            body.append(stage_rows)
-            for k in used_aux:
-                body.append(f'      s_aux{k}[tt_][x_] = ((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_];\n')
-            for k in used_dout:
-                dt = DT_CODE[plan.out_dtypes[k]]
-                nm = f'dout{k}'
-                body.append(f'      s_dy{k}[tt_][x_] = ldf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)});\n')
-            body.append('    }\n')
+        body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
+        body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ') + '    }\n')
 
         def operand_loads(tt, names, state_var):
             code, call = [], []
@@ -702,32 +745,69 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for j in range(len(p.msums)):
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
-        # ---- row loop
-        b.append('  for (int m = 0; m < M; m++) {\n')
-        b.append(f'    const i64 cko = (((i64)bh * nch + ch) * M + m) * {N} + n;\n')
+        # ---- per-row operands of the chunk go through LDS: staged once per row block by the
+        # instance's own lanes (coalesced along m), read back per row as broadcast vectors
+        rowops = []          # (lds name, loader(tt, mexpr) -> expr, register prefix)
+        for i in range(nin):
+            if p.in_names[i] in loop_used and self.in_ext(i) == (True, False) and self.tdep[i]:
+                def ld(tt, mexpr, i=i):
+                    dt = DT_CODE[plan.in_dtypes[i]]
+                    idx = self._in_index(A, i, t=f't0 + {tt}', m=mexpr)
+                    return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
+                rowops.append((f's_c{i}', ld, f'x{i}'))
+        for k in range(naux):
+            if p.aux[k] in loop_used and not is_rowlike(p.aux[k]):
+                rowops.append((f's_ax{k}', (lambda tt, mexpr, k=k: aux_load(k, tt, mexpr)), f'ax{k}'))
+        for k in range(ndaux):
+            if p.daux[k] in loop_used:
+                def ldd(tt, mexpr, k=k):
+                    return f'((const float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + {mexpr}]'
+                rowops.append((f's_da{k}', ldd, f'da{k}'))
+        for k in range(nout):
+            if p.dout_names[k] in loop_used:
+                def ldy(tt, mexpr, k=k):
+                    dt = DT_CODE[plan.out_dtypes[k]]
+                    nmv = f'dout{k}'
+                    return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)(t0 + {tt}) * {A.s(nmv, 1)} + '
+                            f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
+                rowops.append((f's_dy{k}', ldy, f'dy{k}'))
+        MB = 1
+        while MB * 2 <= plan.M and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
+            MB *= 2
+        lanes = min(N, NT)          # lanes of one instance
+        for nm_lds, _, _ in rowops:
+            b.append(f'  __shared__ float {nm_lds}[{IPB}][{MB}][{DT}];\n')
+
+        def ck_index(mexpr):
+            return f'(((i64)bh * nch + ch) * M + ({mexpr})) * {N} + n'
         for k in range(nst):
-            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = ((const float*){A.p(f"sck{k}")})[cko];\n')
-            b.append(f'    float D{k}[1][1]; D{k}[0][0] = ((const float*){A.p(f"dck{k}")})[cko];\n')
+            b.append(f'  float Snx{k} = ((const float*){A.p(f"sck{k}")})[{ck_index("0")}];\n')
+            b.append(f'  float Dnx{k} = ((const float*){A.p(f"dck{k}")})[{ck_index("0")}];\n')
+        b.append(f'  for (int m0 = 0; m0 < M; m0 += {MB}) {{\n')
+        if rowops:
+            b.append('    __syncthreads();\n')
+            b.append(f'    for (int e_ = n; e_ < {MB * DT}; e_ += {lanes}) {{ const int tt_ = e_ / {MB}, mm_ = e_ % {MB}; '
+                     f'const int mc_ = min(m0 + mm_, M - 1);\n')
+            for nm_lds, ld, _ in rowops:
+                b.append(f'      {nm_lds}[inst][mm_][tt_] = {ld("tt_", "mc_")};\n')
+            b.append('    }\n    __syncthreads();\n')
+        b.append(f'  for (int mm = 0; mm < {MB}; mm++) {{\n    const int m = m0 + mm;\n    if (m >= M) break;\n')
+        for k in range(nst):
+            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Snx{k};\n')
+            b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dnx{k};\n')
+        b.append('    { const int mn_ = min(m + 1, M - 1);\n')
+        for k in range(nst):
+            b.append(f'      Snx{k} = ((const float*){A.p(f"sck{k}")})[{ck_index("mn_")}];\n')
+            b.append(f'      Dnx{k} = ((const float*){A.p(f"dck{k}")})[{ck_index("mn_")}];\n')
+        b.append('    }\n')
+        for nm_lds, _, pref in rowops:
+            for tt in range(DT):
+                b.append(f'    float {pref}_{tt}[1][1]; {pref}_{tt}[0][0] = {nm_lds}[inst][mm][{tt}];\n')
         for i in range(nin):
             if p.in_names[i] not in loop_used or not self.in_ext(i)[0]:
                 continue
-            if self.tdep[i]:
-                for tt in range(DT):
-                    b.append(f'    float x{i}_{tt}[1][1]; x{i}_{tt}[0][0] = {load_in(i, tt)};\n')
-            else:
+            if not self.tdep[i]:
                 b.append(f'    float x{i}[1][1]; x{i}[0][0] = {load_in(i, 0)};\n')
-        for k in range(naux):
-            if p.aux[k] in loop_used and not is_rowlike(p.aux[k]):
-                for tt in range(DT):
-                    b.append(f'    float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "m")};\n')
-        for k in range(ndaux):
-            if p.daux[k] in loop_used:
-                for tt in range(DT):
-                    b.append(f'    float da{k}_{tt}[1][1]; da{k}_{tt}[0][0] = {daux_load(k, tt)};\n')
-        for k in range(nout):
-            if p.dout_names[k] in loop_used:
-                for tt in range(DT):
-                    b.append(f'    float dy{k}_{tt}[1][1]; dy{k}_{tt}[0][0] = {dy_load(k, tt)};\n')
 
         def call_args(names, tt, state_var):
             call = []
@@ -781,7 +861,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             nmv = f'din{i}'
             idx = f'(i64)b * {A.s(nmv, 0)} + (i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)} + (i64)n * {A.s(nmv, 4)}'
             b.append(f'    if (valid) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
-        b.append('  }\n')
+        b.append('  }\n  }\n')
         # ---- epilogue
         for tt in range(DT):
             b.append('  {\n')

@@ -145,7 +145,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
     assert _is_pow2(N), f'state width N={N} must be a power of two'
     assert _is_pow2(M), f'state height M={M} must be a power of two'
-    # columns per lane: up to 8 so that a row of up to 128 columns fits one 16-lane DPP row
+    # columns per lane: up to 8, so that a row of up to 128 columns fits one 16-lane DPP row
     C = min(N, 8)
     L = N // C
     while L > 64:
@@ -153,33 +153,34 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256) -> TileConfig:
         L = N // C
     G = 64 // L
     nst = part.nstates + len(part.mat_idx)
-    # rows per lane: bounded by the register budget (state + new state + a few temporaries)
-    R = max(1, min(64 // max(C * nst, 1), 8))
-    R = _pow2_floor(R)
-    # do not give a wave more rows than exist
-    while R > 1 and G * R > M:
+    # rows per lane: bounded by the register budget (state + new state + temporaries) ...
+    R = _pow2_floor(max(1, min(64 // max(C * nst, 1), 8)))
+    while R > 1 and G * R > M:          # ... and by the rows that exist
         R //= 2
-    rows_per_wave = G * R
-    if rows_per_wave > M:
-        # fewer rows than row groups: leave groups idle (handled by row masking)
-        W = 1
-    else:
-        W = max(1, min(4, M // rows_per_wave))
-    # enough workgroups to fill the chip: shrink R while the grid is small
-    def nwg(R_, W_):
-        return B * H * max(1, M // (W_ * G * R_))
-    while R > 1 and nwg(R, W) * W < 4 * n_cu:
+
+    def waves_per_wg(R_):
+        return max(1, min(4, M // (G * R_))) if G * R_ <= M else 1
+
+    def total_waves(R_):
+        W_ = waves_per_wg(R_)
+        return B * H * max(1, -(-M // (W_ * G * R_))) * W_
+
+    # ... and small enough that every SIMD holds at least two waves (latency hiding)
+    while R > 1 and total_waves(R) < 2 * 4 * n_cu:
         R //= 2
-        W = max(1, min(4, M // (G * R)))
-    per_step_regs = 0
-    for i, c in enumerate(part_input_classes(part)):
-        per_step_regs += 1
-    DT = 16
-    if part.dstep_needs_state:
-        DT = 8
+    W = waves_per_wg(R)
+    MT = W * G * R
+    DT = 8 if part.dstep_needs_state else 16
     while DT > 1 and T % DT != 0:
         DT //= 2
-    TS = min(DT, 8)
+    # staging depth: as many timesteps as fit in LDS (inputs + per-row results), at most DT
+    cls = part_input_classes(part)
+    ins = sum({'row': N, 'col': MT, 'scalar': 1, 'mat': 0}[c] for c in cls)
+    per_step = ins + max(part.noutputs + len(part.aux),                                       # forward
+                         len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * MT   # reverse scan
+    TS = DT
+    while TS > 1 and per_step * TS * 4 > 64 * 1024 - 256:
+        TS //= 2
     if part.dstep_needs_state:
         TS = DT
     return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS)
