@@ -1,0 +1,32 @@
+"""Kernel-cache warm-up for the shapes the GPU tests use (called by __graft_entry__.build();
+needs no GPU)."""
+import os
+import sys
+
+import torch as th
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+if HERE not in sys.path:
+    sys.path.insert(0, HERE)
+
+import cases  # noqa: E402
+from flex_rnn_amd import configs, planner, prebuild  # noqa: E402
+from flex_rnn_amd.launch import compile_plan  # noqa: E402
+
+OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn', (2, 32, 2, 32, 16)),
+         ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
+         ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)), ('gla', (1, 16, 1, 16, 16)),
+         ('gla', (1, 32, 1, 16, 16)), ('delta_rule', (2, 32, 2, 16, 16)), ('gated_delta_rule', (2, 32, 2, 16, 16))]
+
+
+def warm(force=False, seen=None):
+    n = 0
+    for name, dims in OTHER:
+        step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)
+        plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
+        n += len(compile_plan(plan, force=force, seen=seen))
+    for name in ('rwkv7', 'gated_delta_rule'):
+        B, T, H, M, N = configs.DEFAULT_DIMS[name]
+        n += len(compile_plan(prebuild.plan_for(name, (B, 128, H, M, N)), force=force, seen=seen))
+    n += len(compile_plan(prebuild.plan_for('rwkv7', (8, 512, 32, 128, 128)), force=force, seen=seen))
+    return n
