@@ -479,7 +479,8 @@ class Emitter:
         colx = (st_ext[0][0], False)
         rrs = R if colx[0] else 1
         g = p.dstep
-        out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux
+        mats = list(p.mat_idx) if p.mat_in_dstep else []
+        out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux + [(True, True)] * len(mats)
         fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>')
         fns = [fn_src]
         used_all = set(used)
@@ -525,6 +526,9 @@ class Emitter:
                 body.append(self._load_const_input(A, i, R, C))
         for i in const_col:
             body.append(f'  float gacc{i}[{rrs}][1];\n#pragma unroll\n  for (int r = 0; r < {rrs}; r++) gacc{i}[r][0] = 0.0f;\n')
+        for i in mats:
+            body.append(f'  float gmacc{i}[{R}][{C}];\n#pragma unroll\n  for (int r = 0; r < {R}; r++)\n#pragma unroll\n'
+                        f'  for (int c = 0; c < {C}; c++) gmacc{i}[r][c] = 0.0f;\n')
         body.append(stg.load(f'T - {TS}', '  '))
         body.append(f'  for (int t0 = T - {TS}; t0 >= 0; t0 -= {TS}) {{\n')
         body.append(f'    if ((t0 + {TS}) % {DT} == 0) {{\n')
@@ -579,7 +583,12 @@ class Emitter:
             for k in range(ndaux):
                 code.append(f'{indent}float da{k}[{rrs}][1];\n')
                 call.append(f'da{k}')
+            for i in mats:
+                code.append(f'{indent}float gm{i}[{R}][{C}];\n')
+                call.append(f'gm{i}')
             code.append(f'{indent}bw_dstep(' + ', '.join(call) + ');\n')
+            for i in mats:
+                code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {R}; r++)\n#pragma unroll\n{indent}for (int c = 0; c < {C}; c++) gmacc{i}[r][c] += gm{i}[r][c];\n')
             for k in range(nst):
                 rr, cc = _dims(st_ext[k], R, C)
                 code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {rr}; r++)\n#pragma unroll\n{indent}for (int c = 0; c < {cc}; c++) D{k}[r][c] = nD{k}[r][c];\n')
@@ -641,6 +650,14 @@ class Emitter:
             nm = f'din{i}'
             body.append(f'  if (l == 0) {{\n#pragma unroll\n    for (int r = 0; r < {R}; r++) if (row0 + r < M) '
                         f'atomic_addf({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 2)} + (i64)(row0 + r) * {A.s(nm, 3)}, gacc{i}[{"r" if rrs > 1 else "0"}][0]);\n  }}\n')
+        for i in mats:
+            nm = f'din{i}'
+            bB, _, bH = plan.in_bcast[i]
+            idx = (f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 2)} + (i64)(row0 + r) * {A.s(nm, 3)} + (i64)COL(c) * {A.s(nm, 4)}')
+            put = (f'atomic_addf({A.p(nm)}, {idx}, gmacc{i}[r][c])' if (bB or bH)
+                   else f'stf<0>({A.p(nm)}, {idx}, gmacc{i}[r][c])')
+            body.append(f'#pragma unroll\n  for (int r = 0; r < {R}; r++) if (row0 + r < M) {{\n#pragma unroll\n'
+                        f'    for (int c = 0; c < {C}; c++) {put}; }}\n')
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
             dt = DT_CODE[plan.st_dtypes[k]]
@@ -659,6 +676,8 @@ class Emitter:
         N, DT = plan.N, t.DT
         IPB = max(1, 64 // N)
         NT = max(64, N)
+        HB = max(1, getattr(t, 'HB', 1))
+        assert plan.H % HB == 0
         A = _Args()
         nin, nst, nout = p.ninputs, p.nstates, p.noutputs
         naux, ndaux = len(p.aux), len(p.daux)
@@ -667,7 +686,8 @@ class Emitter:
         rs = p.row_idx + p.scalar_idx
         red = f'inst_allreduce<{N}>'
         op_names = [nm_[m].args[0] for m in p.msums]
-        drow_exts = st_ext + [(True, True)] * len(p.mat_idx) + [self.jext[o] for o in op_names]
+        mats2 = [] if p.mat_in_dstep else list(p.mat_idx)
+        drow_exts = st_ext + [(True, True)] * len(mats2) + [self.jext[o] for o in op_names]
         drow_src, drow_used = emit_graph_fn(p.drow, 'bw_drow', 1, 1, drow_exts, red)
         re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', 1, 1, st_ext, red)
         epi_exts = [self.in_ext(i) for i in rs]
@@ -703,9 +723,22 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   int ch = blockIdx.x * {IPB} + inst;
   const bool valid = ch < nch;
   if (!valid) ch = nch - 1;
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const int HG = H / {HB};                     // head groups; an instance walks {HB} heads
+  const int b = blockIdx.y / HG, h0 = (blockIdx.y % HG) * {HB};
   const int t0 = ch * {DT};
 ''')
+        # gradients of inputs broadcast over heads / time are summed in registers across the
+        # head loop / the chunk before they leave the kernel
+        def bflags(i):
+            return plan.in_bcast[i]
+        hacc = [i for i in rs if bflags(i)[2] and HB > 1]
+        for i in hacc:
+            if bflags(i)[1]:
+                b.append(f'  float gh{i} = 0.0f;\n')
+            else:
+                for tt in range(DT):
+                    b.append(f'  float gh{i}_{tt} = 0.0f;\n')
+        b.append(f'  for (int hh = 0; hh < {HB}; hh++) {{\n  const int h = h0 + hh; const int bh = b * H + h;\n')
 
         def load_in(i, tt, m=None):
             ext = self.in_ext(i)
@@ -835,7 +868,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                 b.append(f'    float Sh{k}_{tt + 1}[1][1];\n')
             call = call_args(re_used, tt, lambda k, tt=tt: f'Sh{k}_{tt}') + [f'Sh{k}_{tt + 1}' for k in range(nst)]
             b.append('    bw_restep(' + ', '.join(call) + ');\n')
-        for i in p.mat_idx:
+        for i in mats2:
             b.append(f'    float ma{i} = 0.0f;\n')
         for tt in range(DT - 1, -1, -1):
             b.append('    {\n')
@@ -843,7 +876,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             for k in range(nst):
                 b.append(f'      float nD{k}[1][1];\n')
                 call.append(f'nD{k}')
-            for i in p.mat_idx:
+            for i in mats2:
                 b.append(f'      float gm{i}[1][1];\n')
                 call.append(f'gm{i}')
             for j in range(len(p.msums)):
@@ -852,17 +885,37 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append('      bw_drow(' + ', '.join(call) + ');\n')
             for k in range(nst):
                 b.append(f'      D{k}[0][0] = nD{k}[0][0];\n')
-            for i in p.mat_idx:
+            for i in mats2:
                 b.append(f'      ma{i} += gm{i}[0][0];\n')
             for j in range(len(p.msums)):
                 b.append(f'      acc{j}_{tt} += op{j}[0][0];\n')
             b.append('    }\n')
-        for i in p.mat_idx:
+        for i in mats2:
             nmv = f'din{i}'
             idx = f'(i64)b * {A.s(nmv, 0)} + (i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)} + (i64)n * {A.s(nmv, 4)}'
             b.append(f'    if (valid) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
         b.append('  }\n  }\n')
         # ---- epilogue
+        def out_index(i, tt, hexpr):
+            nmv = f'din{i}'
+            ext = self.in_ext(i)
+            return (f'(i64)b * {A.s(nmv, 0)} + (i64)(t0 + {tt}) * {A.s(nmv, 1)} + (i64)({hexpr}) * {A.s(nmv, 2)}'
+                    + (f' + (i64)n * {A.s(nmv, 4)}' if ext[1] else ''))
+
+        def write_out(i, tt, hexpr, val, ind):
+            nmv = f'din{i}'
+            ext = self.in_ext(i)
+            bB, bT, bH = bflags(i)
+            cond = 'valid' + ('' if ext[1] else ' && n == 0')
+            idx = out_index(i, tt, hexpr)
+            if bB or bT or (bH and HB < plan.H):
+                return f'{ind}if ({cond}) atomic_addf({A.p(nmv)}, {idx}, {val});\n'
+            dt = 0 if i in self.atomic else DT_CODE[plan.in_dtypes[i]]      # broadcast inputs use fp32 scratch
+            return f'{ind}if ({cond}) stf<{dt}>({A.p(nmv)}, {idx}, {val});\n'
+
+        tacc = [i for i in rs if bflags(i)[1]]
+        for i in tacc:
+            b.append(f'  float gt{i} = 0.0f;\n')
         for tt in range(DT):
             b.append('  {\n')
             for j, mname in enumerate(p.msums):
@@ -878,17 +931,25 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                 call.append(f'g{i}')
             b.append('    bw_epi(' + ', '.join(call) + ');\n')
             for i in rs:
-                nmv = f'din{i}'
-                ext = self.in_ext(i)
-                tterm = f'(i64)(t0 + {tt}) * {A.s(nmv, 1)}'
-                idx = f'(i64)b * {A.s(nmv, 0)} + {tterm} + (i64)h * {A.s(nmv, 2)}' + (f' + (i64)n * {A.s(nmv, 4)}' if ext[1] else '')
-                cond = 'valid' + ('' if ext[1] else ' && n == 0')
-                if i in self.atomic:
-                    b.append(f'    if ({cond}) atomic_addf({A.p(nmv)}, {idx}, g{i}[0][0]);\n')
+                if i in tacc:
+                    b.append(f'    gt{i} += g{i}[0][0];\n')
+                elif i in hacc:
+                    b.append(f'    gh{i}_{tt} += g{i}[0][0];\n')
                 else:
-                    dt = DT_CODE[plan.in_dtypes[i]]
-                    b.append(f'    if ({cond}) stf<{dt}>({A.p(nmv)}, {idx}, g{i}[0][0]);\n')
+                    b.append(write_out(i, tt, 'h', f'g{i}[0][0]', '    '))
             b.append('  }\n')
+        for i in tacc:
+            if i in hacc:
+                b.append(f'  gh{i} += gt{i};\n')
+            else:
+                b.append(write_out(i, '0', 'h', f'gt{i}', '  '))
+        b.append('  }\n')        # head loop
+        for i in hacc:
+            if i in tacc:
+                b.append(write_out(i, '0', 'h0', f'gh{i}', '  '))
+            else:
+                for tt in range(DT):
+                    b.append(write_out(i, tt, 'h0', f'gh{i}_{tt}', '  '))
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
         source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + kernel
-        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', 'B * H', '1'))
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})', '1'))

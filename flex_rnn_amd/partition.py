@@ -63,6 +63,7 @@ class Partition:
     drow: Graph = None
     epi: Graph = None
     dstep_needs_state: bool = False
+    mat_in_dstep: bool = False       # matrix-input grads are accumulated by the reverse scan (it has the state)
 
     def describe(self) -> str:
         return '\n\n'.join(g.code() for g in (self.fw, self.restep, self.dstep, self.drow, self.epi))
@@ -152,8 +153,17 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
         if mdep[v]:
             raise PartitionError('nested reductions over the row axis are not supported')
 
+    # --- where matrix-input gradients are formed ------------------------------------------
+    # If the reverse scan has to recompute the state anyway (a column gradient or a saved
+    # backward sum reads it), it also accumulates the matrix-input gradients over the whole
+    # sequence in registers; otherwise the gradient kernel does, chunk by chunk.
+    probe = joint.extract('probe', list(dst_names) + [din_names[i] for i in col_idx], cut=set(aux_all))
+    mat_in_dstep = bool(mat_idx) and any(probe.uses(s_) for s_ in st_names)
+    mats_drow = [] if mat_in_dstep else list(mat_idx)
+    mats_dstep = list(mat_idx) if mat_in_dstep else []
+
     # --- drow: per-element part of the gradient kernel -------------------------------
-    drow_outs = list(dst_names) + [din_names[i] for i in mat_idx] + msum_operands
+    drow_outs = list(dst_names) + [din_names[i] for i in mats_drow] + msum_operands
     for v in list(dst_names) + [din_names[i] for i in mat_idx + col_idx]:
         if mdep.get(v, False):
             raise PartitionError('state / column / matrix gradient depends on a reduction over the row axis')
@@ -163,7 +173,7 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
     daux = [s for s in bsum_n if drow.uses(s)]
 
     # --- dstep: reverse scan -----------------------------------------------------------
-    dstep_outs = list(dst_names) + [din_names[i] for i in col_idx] + daux
+    dstep_outs = list(dst_names) + [din_names[i] for i in col_idx] + daux + [din_names[i] for i in mats_dstep]
     dstep = joint.extract('dstep', dstep_outs, cut=set(aux_all))
     for n in dstep.nodes:
         if n.op == 'sum' and n.dims != (1,):
@@ -192,5 +202,5 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
                   out_names, nst_names, din_names, dst_names, aux, daux, msums,
                   col_idx, row_idx, scalar_idx, mat_idx,
                   fw=fw, restep=restep, dstep=dstep, drow=drow, epi=epi,
-                  dstep_needs_state=dstep_needs_state)
+                  dstep_needs_state=dstep_needs_state, mat_in_dstep=mat_in_dstep)
     return p

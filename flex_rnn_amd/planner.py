@@ -15,6 +15,7 @@ The kernels, their tiling and the layout of the hidden buffers (`state_store`,
 from __future__ import annotations
 
 import hashlib
+import os
 from dataclasses import dataclass, field
 from typing import Callable, Dict, List, Optional, Sequence, Tuple
 
@@ -79,6 +80,7 @@ class TileConfig:
     TS: int
     R1: int = 0          # rows per lane / waves in bw1 (0 = same as fw)
     W1: int = 0
+    HB: int = 1          # heads walked by one gradient-kernel instance (sums head-broadcast grads in registers)
 
     @property
     def G(self): return 64 // self.L
@@ -141,7 +143,7 @@ def classify(inputs, state):
     return dims, cls, bcast
 
 
-def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256) -> TileConfig:
+def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
     assert _is_pow2(N), f'state width N={N} must be a power of two'
     assert _is_pow2(M), f'state height M={M} must be a power of two'
@@ -183,7 +185,16 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256) -> TileConfig:
         TS //= 2
     if part.dstep_needs_state:
         TS = DT
-    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS)
+    # gradient kernel: walk several heads per instance when a row/scalar input is shared by all
+    # heads (its gradient then needs no atomics inside the group), keeping >= 2 waves per SIMD
+    HB = 1
+    if in_bcast is not None and any(in_bcast[i][2] for i in part.row_idx + part.scalar_idx):
+        ipb = max(1, 64 // N)
+        waves = lambda hb: B * (H // hb) * -(-(T // DT) // ipb) * max(1, N // 64)
+        HB = H & -H                     # largest power of two dividing H
+        while HB > 1 and waves(HB) < 2 * 4 * n_cu:
+            HB //= 2
+    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, HB=HB)
 
 
 def part_input_classes(part: Partition) -> List[str]:
@@ -212,7 +223,11 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
     part = partition(joint, ninputs, nstates, noutputs, cls)
 
     if tile is None:
-        tile = choose_tiles(B, T, H, M, N, part)
+        tile = choose_tiles(B, T, H, M, N, part, in_bcast=bcast)
+        override = os.environ.get('FLEX_RNN_TILE')          # e.g. "R=2,TS=8" (tuning / tests)
+        if override:
+            import dataclasses
+            tile = dataclasses.replace(tile, **{k: int(v) for k, v in (kv.split('=') for kv in override.split(','))})
     assert T % tile.DT == 0 and tile.DT % tile.TS == 0
     nchunks = T // tile.DT
     plan = Plan(B, T, H, M, N, part, cls, [i.dtype for i in inputs], bcast,

@@ -109,6 +109,7 @@ def run_plan(part, inputs: Sequence[torch.Tensor], states: Sequence[torch.Tensor
         return hist
 
     D = [d.to(dtype) for d in dstatesT]
+    dmat = {i: torch.zeros(B, H, M, N, dtype=dtype) for i in part.mat_idx}
     dck = [None] * (T // DT)
     dcol = {i: [None] * T for i in part.col_idx}
     daux_hist = [None] * T
@@ -128,14 +129,17 @@ def run_plan(part, inputs: Sequence[torch.Tensor], states: Sequence[torch.Tensor
         D = [d.expand(B, H, M, N) for d in res[:nst]]
         for k, i in enumerate(part.col_idx):
             dcol[i][t] = res[nst + k].expand(B, H, M, 1)
-        daux_hist[t] = res[nst + len(part.col_idx):]
+        daux_hist[t] = res[nst + len(part.col_idx):nst + len(part.col_idx) + ndaux]
+        if part.mat_in_dstep:
+            for k, i in enumerate(part.mat_idx):
+                dmat[i] = dmat[i] + res[nst + len(part.col_idx) + ndaux + k].expand(B, H, M, N)
     dstate0 = tuple(D)
 
     # ------------------------------------------------------------------ gradient pass
     nm = part.joint.node_map()
     rs = part.row_idx + part.scalar_idx
     drs = {i: [None] * T for i in rs}
-    dmat = {i: torch.zeros(B, H, M, N, dtype=dtype) for i in part.mat_idx}
+    mats_drow = [] if part.mat_in_dstep else list(part.mat_idx)
     for c in range(T // DT):
         hist = recompute_chunk(c)
         D = dck[c]
@@ -148,9 +152,9 @@ def run_plan(part, inputs: Sequence[torch.Tensor], states: Sequence[torch.Tensor
             env.update(dict(zip(part.dnst_names, D)))
             res = eval_graph(part.drow, env, dtype)
             D = [d.expand(B, H, M, N) for d in res[:nst]]
-            for k, i in enumerate(part.mat_idx):
+            for k, i in enumerate(mats_drow):
                 dmat[i] = dmat[i] + res[nst + k].expand(B, H, M, N)
-            ops = res[nst + len(part.mat_idx):]
+            ops = res[nst + len(mats_drow):]
             # accumulate the sums over the row axis, then run the epilogue
             eenv = bind_inputs(part.epi, t)
             eenv.update(dict(zip(part.aux, aux_hist[t])))
