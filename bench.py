@@ -37,6 +37,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--workload', default='rwkv7', choices=sorted(WORK))
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run one plain 1 GiB device copy (reference dispatch for HBM byte counters)')
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this build measures one GPU; --gpus {args.gpus} is not supported '
@@ -93,15 +95,27 @@ def main():
     achieved = kflop[dominant] * elems / (kavg[dominant] * 1e-3) / 1e12
     gpu_ms = sum(kavg.values())
     step_tflops = (w['flop_fwd'] + w['flop_bwd']) * elems / (gpu_ms * 1e-3) / 1e12
+    traffic = None        # HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc runs
+    tpath = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+    if os.path.isfile(tpath):
+        rec = json.load(open(tpath)).get(name, {}).get(dominant)
+        if rec:
+            traffic = round(rec['read_bytes'] + rec['write_bytes'])
     roofline = {
         'bound': 'valu', 'kernel': dominant, 'achieved': round(achieved, 3), 'peak': PEAK_FP32_TFLOPS,
-        'unit': 'TFLOP/s', 'frac': round(achieved / PEAK_FP32_TFLOPS, 4), 'traffic': None,
+        'unit': 'TFLOP/s', 'frac': round(achieved / PEAK_FP32_TFLOPS, 4), 'traffic': traffic,
         'kernel_ms': {k: round(v, 4) for k, v in kavg.items()},
         'step_achieved': round(step_tflops, 3), 'step_frac': round(step_tflops / PEAK_FP32_TFLOPS, 4),
         'hbm_GBps_algorithmic': round(w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9, 1),
         'hbm_frac': round(w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
     }
 
+    if args.calibrate_copy:
+        src = th.empty(1 << 28, dtype=th.float32, device=dev).normal_()
+        dst = th.empty_like(src)
+        dst.copy_(src)                      # reads 1 GiB, writes 1 GiB
+        th.cuda.synchronize()
+        del src, dst
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(name)
