@@ -225,22 +225,35 @@ class _Stager:
     """Global -> LDS staging of per-timestep operands for TS timesteps, split in two phases so
     that the loads of the next chunk are in flight while the current one is computed:
     `load(t0)` issues every load of the chunk back to back into registers (raw bits),
-    `write()` converts them to fp32 and stores them to LDS."""
+    `write()` converts them to fp32 and stores them to LDS.  Element e = tid + it*NT of the
+    [TS][ln] tile is (timestep e / ln, position e % ln); when NT is a multiple of ln the position
+    is the same for every `it`, so one 64-bit base index per operand is computed up front
+    (`bases()`) and each load adds a multiple of the operand's time stride."""
 
     def __init__(self, TS: int, NT: int):
         self.TS, self.NT = TS, NT
-        self.items = []          # (lds name, row length, dtype code, pointer expr, index fn(t0, tt_, x_))
+        self.items = []      # (lds name, row length, dtype code, pointer, index fn(tt_, x_) at t0 = 0, time stride)
 
-    def add(self, name, ln, dt, ptr, idx_fn):
-        self.items.append((name, ln, dt, ptr, idx_fn))
+    def add(self, name, ln, dt, ptr, idx_fn, tstride):
+        self.items.append((name, ln, dt, ptr, idx_fn, tstride))
 
     def _iters(self, ln):
         return (self.TS * ln + self.NT - 1) // self.NT
 
+    def _linear(self, ln):
+        return self.NT % ln == 0
+
     def decls(self) -> str:
         out = ''
-        for name, ln, dt, ptr, fn in self.items:
+        for name, ln, dt, ptr, fn, ts in self.items:
             out += f'  __shared__ float {name}[{self.TS}][{ln}];\n  unsigned pf_{name}[{self._iters(ln)}];\n'
+        return out
+
+    def bases(self) -> str:
+        out = ''
+        for name, ln, dt, ptr, fn, ts in self.items:
+            if self._linear(ln):
+                out += f'  const i64 pb_{name} = {fn(f"(tid / {ln})", f"(tid % {ln})")};\n'
         return out
 
     def _loop(self, ln, body, ind):
@@ -251,13 +264,17 @@ class _Stager:
 
     def load(self, t0: str, ind: str) -> str:
         out = ''
-        for name, ln, dt, ptr, fn in self.items:
-            out += self._loop(ln, f'pf_{name}[it_] = ldr<{dt}>({ptr}, {fn(t0, "tt_", "x_")});', ind)
+        for name, ln, dt, ptr, fn, ts in self.items:
+            if self._linear(ln):
+                idx = f'pb_{name} + (i64)(({t0}) + it_ * {self.NT // ln}) * {ts}'
+            else:
+                idx = f'{fn("tt_", "x_")} + (i64)({t0}) * {ts}'
+            out += self._loop(ln, f'pf_{name}[it_] = ldr<{dt}>({ptr}, {idx});', ind)
         return out
 
     def write(self, ind: str) -> str:
         out = ''
-        for name, ln, dt, ptr, fn in self.items:
+        for name, ln, dt, ptr, fn, ts in self.items:
             out += self._loop(ln, f'{name}[tt_][x_] = cvr<{dt}>(pf_{name}[it_]);', ind)
         return out
 
@@ -322,13 +339,14 @@ class Emitter:
         ext = self.in_ext(i)
         N = self.plan.N
         dt = DT_CODE[self.plan.in_dtypes[i]]
+        ts = A.s(f'in{i}', 1)
         if ext == (False, True):
-            st.add(f's_in{i}', N, dt, A.p(f'in{i}'), lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}', n=x))
+            st.add(f's_in{i}', N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x), ts)
         elif ext == (True, False):
             st.add(f's_in{i}', MT, dt, A.p(f'in{i}'),
-                   lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}', m=f'min(mt * {MT} + {x}, M - 1)'))
+                   lambda tt, x, i=i: self._in_index(A, i, t=tt, m=f'min(mt * {MT} + {x}, M - 1)'), ts)
         else:
-            st.add(f's_in{i}', 1, dt, A.p(f'in{i}'), lambda t0, tt, x, i=i: self._in_index(A, i, t=f'{t0} + {tt}'))
+            st.add(f's_in{i}', 1, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt), ts)
 
     def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str) -> str:
         """Registers <- staged LDS operand for timestep tt."""
@@ -378,7 +396,7 @@ class Emitter:
         for i in used_in:
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
-        body.append(stg.decls())
+        body.append(stg.decls() + stg.bases())
         for k in range(nout):
             body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
         for k in range(naux):
@@ -500,13 +518,13 @@ class Emitter:
                 self._stage_input(stg, A, i, MT)
         for k in used_aux:
             stg.add(f's_aux{k}', MT, 0, A.p('aux'),
-                    lambda t0, tt, x, k=k: f'((((i64){k} * A.B + b) * H + h) * T + ({t0} + {tt})) * M + min(mt * {MT} + {x}, M - 1)')
+                    lambda tt, x, k=k: f'((((i64){k} * A.B + b) * H + h) * T + {tt}) * M + min(mt * {MT} + {x}, M - 1)', 'M')
         for k in used_dout:
             nm = f'dout{k}'
             stg.add(f's_dy{k}', MT, DT_CODE[plan.out_dtypes[k]], A.p(nm),
-                    lambda t0, tt, x, nm=nm: (f'(i64)b * {A.s(nm, 0)} + (i64)({t0} + {tt}) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + '
-                                               f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'))
-        body.append(stg.decls())
+                    lambda tt, x, nm=nm: (f'(i64)b * {A.s(nm, 0)} + (i64)({tt}) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + '
+                                           f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'), A.s(nm, 1))
+        body.append(stg.decls() + stg.bases())
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
         for i in tdep_col:
@@ -811,11 +829,11 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for nm_lds, _, _ in rowops:
             b.append(f'  __shared__ float {nm_lds}[{IPB}][{MB}][{DT}];\n')
 
-        def ck_index(mexpr):
-            return f'(((i64)bh * nch + ch) * M + ({mexpr})) * {N} + n'
+        # element (row m, column n) of this instance's checkpoint: base pointer + m * N
         for k in range(nst):
-            b.append(f'  float Snx{k} = ((const float*){A.p(f"sck{k}")})[{ck_index("0")}];\n')
-            b.append(f'  float Dnx{k} = ((const float*){A.p(f"dck{k}")})[{ck_index("0")}];\n')
+            b.append(f'  const float* sckp{k} = (const float*){A.p(f"sck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
+            b.append(f'  const float* dckp{k} = (const float*){A.p(f"dck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
+            b.append(f'  float Snx{k} = sckp{k}[0];\n  float Dnx{k} = dckp{k}[0];\n')
         b.append(f'  for (int m0 = 0; m0 < M; m0 += {MB}) {{\n')
         if rowops:
             b.append('    __syncthreads();\n')
@@ -830,8 +848,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dnx{k};\n')
         b.append('    { const int mn_ = min(m + 1, M - 1);\n')
         for k in range(nst):
-            b.append(f'      Snx{k} = ((const float*){A.p(f"sck{k}")})[{ck_index("mn_")}];\n')
-            b.append(f'      Dnx{k} = ((const float*){A.p(f"dck{k}")})[{ck_index("mn_")}];\n')
+            b.append(f'      Snx{k} = sckp{k}[mn_ * {N}];\n')
+            b.append(f'      Dnx{k} = dckp{k}[mn_ * {N}];\n')
         b.append('    }\n')
         for nm_lds, _, pref in rowops:
             for tt in range(DT):
