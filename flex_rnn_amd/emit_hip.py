@@ -228,11 +228,12 @@ class _Stager:
     `write()` converts them to fp32 and stores them to LDS.  Element e = tid + it*NT of the
     [TS][ln] tile is (timestep e / ln, position e % ln); when NT is a multiple of ln the position
     is the same for every `it`, so one 64-bit base index per operand is computed up front
-    (`bases()`) and each load adds a multiple of the operand's time stride."""
+    (`bases()`) and each load adds a multiple of the operand's time stride.  With `tail` the
+    timestep is clamped to T-1 (the last chunk may be partial; the surplus values are unused)."""
 
-    def __init__(self, TS: int, NT: int):
-        self.TS, self.NT = TS, NT
-        self.items = []      # (lds name, row length, dtype code, pointer, index fn(tt_, x_) at t0 = 0, time stride)
+    def __init__(self, TS: int, NT: int, tail: bool = False):
+        self.TS, self.NT, self.tail = TS, NT, tail
+        self.items = []      # (lds name, row length, dtype code, pointer, index fn(t, x_), time stride)
 
     def add(self, name, ln, dt, ptr, idx_fn, tstride):
         self.items.append((name, ln, dt, ptr, idx_fn, tstride))
@@ -253,7 +254,7 @@ class _Stager:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
             if self._linear(ln):
-                out += f'  const i64 pb_{name} = {fn(f"(tid / {ln})", f"(tid % {ln})")};\n'
+                out += f'  const i64 pb_{name} = {fn("0", f"(tid % {ln})")};\n  const int tb_{name} = tid / {ln};\n'
         return out
 
     def _loop(self, ln, body, ind):
@@ -262,13 +263,17 @@ class _Stager:
         return (f'#pragma unroll\n{ind}for (int it_ = 0; it_ < {self._iters(ln)}; it_++) {{ const int e_ = tid + it_ * {self.NT}; '
                 f'const int tt_ = e_ / {ln}, x_ = e_ % {ln}; (void)tt_; (void)x_; {guard}{body} }}\n')
 
+    def _clamp(self, t):
+        return f'min({t}, T - 1)' if self.tail else t
+
     def load(self, t0: str, ind: str) -> str:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
             if self._linear(ln):
-                idx = f'pb_{name} + (i64)(({t0}) + it_ * {self.NT // ln}) * {ts}'
+                t = self._clamp(f'({t0}) + tb_{name} + it_ * {self.NT // ln}')
+                idx = f'pb_{name} + (i64)({t}) * {ts}'
             else:
-                idx = f'{fn("tt_", "x_")} + (i64)({t0}) * {ts}'
+                idx = fn(self._clamp(f'({t0}) + tt_'), 'x_')
             out += self._loop(ln, f'pf_{name}[it_] = ldr<{dt}>({ptr}, {idx});', ind)
         return out
 
@@ -300,6 +305,9 @@ class Emitter:
         self.tdep = [(plan.T == 1 or not b[1]) and c != 'mat' for b, c in zip(plan.in_bcast, self.cls)]
         self.atomic = set(plan.atomic)
         self.jext = p.joint.ext_table()
+        # the last chunk is partial when T is not a multiple of the chunk sizes; the guards that
+        # handles it are only emitted then, so aligned lengths keep the unguarded code
+        self.tail_dt = plan.T % plan.tile.DT != 0
 
     # ------------------------------------------------------------------ helpers
     def in_ext(self, i: int):
@@ -392,7 +400,8 @@ class Emitter:
         src, MT = self._row_kernel_common(A, used_in, R, W)
         body = []
         # staging buffers
-        stg = _Stager(TS, NT)
+        tail = plan.T % TS != 0
+        stg = _Stager(TS, NT, tail)
         for i in used_in:
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
@@ -425,7 +434,8 @@ class Emitter:
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
         body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
-        body.append(f'#pragma unroll 2\n    for (int tt = 0; tt < {TS}; tt++) {{\n')
+        body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
+        body.append(f'#pragma unroll 2\n    for (int tt = 0; tt < nt; tt++) {{\n')
         call = []
         for nm_ in used:
             if nm_ in p.in_names:
@@ -460,7 +470,7 @@ class Emitter:
         body.append('      }\n    }\n    __syncthreads();\n')
         # flush
         body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
-                    f'      if (m_ < M) {{\n')
+                    f'      if (m_ < M && tt_ < nt) {{\n')
         for k in range(nout):
             dt = DT_CODE[plan.out_dtypes[k]]
             nm = f'out{k}'
@@ -512,7 +522,8 @@ class Emitter:
         used_dout = [k for k in range(nout) if p.dout_names[k] in used_all]
         src, MT = self._row_kernel_common(A, used_in, R, W)
         body = []
-        stg = _Stager(TS, NT)
+        tail = plan.T % TS != 0
+        stg = _Stager(TS, NT, tail)
         for i in used_in:
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
@@ -547,14 +558,16 @@ class Emitter:
         for i in mats:
             body.append(f'  float gmacc{i}[{R}][{C}];\n#pragma unroll\n  for (int r = 0; r < {R}; r++)\n#pragma unroll\n'
                         f'  for (int c = 0; c < {C}; c++) gmacc{i}[r][c] = 0.0f;\n')
-        body.append(stg.load(f'T - {TS}', '  '))
-        body.append(f'  for (int t0 = T - {TS}; t0 >= 0; t0 -= {TS}) {{\n')
-        body.append(f'    if ((t0 + {TS}) % {DT} == 0) {{\n')
+        body.append(f'  const int tlast = ((T - 1) / {TS}) * {TS};\n')
+        body.append(stg.load('tlast', '  '))
+        body.append(f'  for (int t0 = tlast; t0 >= 0; t0 -= {TS}) {{\n')
+        body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
+        body.append(f'    if ((t0 + {TS}) % {DT} == 0{f" || t0 + {TS} >= T" if self.tail_dt else ""}) {{\n')
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
             body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
-                        f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"(t0 + {TS}) / {DT} - 1")}] = D{k}[r][c]; }}\n')
+                        f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"t0 / {DT}")}] = D{k}[r][c]; }}\n')
         body.append('    }\n    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
@@ -622,7 +635,7 @@ class Emitter:
             return code
 
         if not needs_state:
-            body.append(f'#pragma unroll 2\n    for (int tt = {TS - 1}; tt >= 0; tt--) {{\n')
+            body.append(f'#pragma unroll 2\n    for (int tt = nt - 1; tt >= 0; tt--) {{\n')
             body += dstep_block('tt', lambda k: (_ for _ in ()).throw(AssertionError()))
             body.append('    }\n')
         else:
@@ -637,21 +650,21 @@ class Emitter:
                     rr, cc = _dims(st_ext[k], R, C)
                     body.append(f'    float Sh{k}_{tt}[{rr}][{cc}];\n')
             for tt in range(DT - 1):
-                body.append('    {\n')
+                body.append(f'    if ({tt + 1} < nt) {{\n' if tail else '    {\n')
                 code, call = operand_loads(str(tt), re_used, lambda k, tt=tt: f'Sh{k}_{tt}')
                 body += code
                 for k in range(nst):
                     call.append(f'Sh{k}_{tt + 1}')
                 body.append('      bw_restep(' + ', '.join(call) + ');\n    }\n')
             for tt in range(DT - 1, -1, -1):
-                body.append('    {\n')
+                body.append(f'    if ({tt} < nt) {{\n' if tail else '    {\n')
                 body += dstep_block(str(tt), lambda k, tt=tt: f'Sh{k}_{tt}')
                 body.append('    }\n')
         body.append('    __syncthreads();\n')
         # flush column grads and daux
         if tdep_col or ndaux:
             body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
-                        f'      if (m_ < M) {{\n')
+                        f'      if (m_ < M && tt_ < nt) {{\n')
             for i in tdep_col:
                 nm = f'din{i}'
                 idx = f'(i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}'
@@ -744,7 +757,14 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   const int HG = H / {HB};                     // head groups; an instance walks {HB} heads
   const int b = blockIdx.y / HG, h0 = (blockIdx.y % HG) * {HB};
   const int t0 = ch * {DT};
+  const int nt = {f"min({DT}, T - t0)" if self.tail_dt else DT};          // timesteps of this chunk
+  (void)nt;
 ''')
+        tail = self.tail_dt
+
+        def tclamp(tt):
+            return f'min(t0 + {tt}, T - 1)' if tail else f't0 + {tt}'
+
         # gradients of inputs broadcast over heads / time are summed in registers across the
         # head loop / the chunk before they leave the kernel
         def bflags(i):
@@ -761,7 +781,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         def load_in(i, tt, m=None):
             ext = self.in_ext(i)
             dt = DT_CODE[plan.in_dtypes[i]]
-            idx = self._in_index(A, i, t=(f't0 + {tt}' if self.tdep[i] else '0'),
+            idx = self._in_index(A, i, t=(tclamp(tt) if self.tdep[i] else '0'),
                                  m=('m' if ext[0] else None), n=('n' if ext[1] else None))
             return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
 
@@ -769,16 +789,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             return f'x{i}_{tt}' if self.tdep[i] else f'x{i}'
 
         def aux_load(k, tt, mexpr):
-            return f'((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + {mexpr}]'
-
-        def daux_load(k, tt):
-            return f'((const float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + m]'
-
-        def dy_load(k, tt):
-            dt = DT_CODE[plan.out_dtypes[k]]
-            nmv = f'dout{k}'
-            return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)(t0 + {tt}) * {A.s(nmv, 1)} + '
-                    f'(i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)})')
+            return f'((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + ({tclamp(tt)})) * M + {mexpr}]'
 
         # ---- per-chunk loads of everything without a row extent
         for i in range(nin):
@@ -803,7 +814,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             if p.in_names[i] in loop_used and self.in_ext(i) == (True, False) and self.tdep[i]:
                 def ld(tt, mexpr, i=i):
                     dt = DT_CODE[plan.in_dtypes[i]]
-                    idx = self._in_index(A, i, t=f't0 + {tt}', m=mexpr)
+                    idx = self._in_index(A, i, t=tclamp(tt), m=mexpr)
                     return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
                 rowops.append((f's_c{i}', ld, f'x{i}'))
         for k in range(naux):
@@ -812,14 +823,14 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for k in range(ndaux):
             if p.daux[k] in loop_used:
                 def ldd(tt, mexpr, k=k):
-                    return f'((const float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + {tt})) * M + {mexpr}]'
+                    return f'((const float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + ({tclamp(tt)})) * M + {mexpr}]'
                 rowops.append((f's_da{k}', ldd, f'da{k}'))
         for k in range(nout):
             if p.dout_names[k] in loop_used:
                 def ldy(tt, mexpr, k=k):
                     dt = DT_CODE[plan.out_dtypes[k]]
                     nmv = f'dout{k}'
-                    return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)(t0 + {tt}) * {A.s(nmv, 1)} + '
+                    return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)({tclamp(tt)}) * {A.s(nmv, 1)} + '
                             f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
                 rowops.append((f's_dy{k}', ldy, f'dy{k}'))
         MB = 1
@@ -889,7 +900,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for i in mats2:
             b.append(f'    float ma{i} = 0.0f;\n')
         for tt in range(DT - 1, -1, -1):
-            b.append('    {\n')
+            b.append(f'    if ({tt} < nt) {{\n' if tail else '    {\n')
             call = call_args(drow_used, tt, lambda k, tt=tt: f'Sh{k}_{tt}')
             for k in range(nst):
                 b.append(f'      float nD{k}[1][1];\n')
@@ -925,6 +936,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             ext = self.in_ext(i)
             bB, bT, bH = bflags(i)
             cond = 'valid' + ('' if ext[1] else ' && n == 0')
+            if tail and not bT:
+                cond += f' && t0 + {tt} < T'
             idx = out_index(i, tt, hexpr)
             if bB or bT or (bH and HB < plan.H):
                 return f'{ind}if ({cond}) atomic_addf({A.p(nmv)}, {idx}, {val});\n'

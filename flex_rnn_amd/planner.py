@@ -173,7 +173,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     W = waves_per_wg(R)
     MT = W * G * R
     DT = 8 if part.dstep_needs_state else 16
-    while DT > 1 and T % DT != 0:
+    while DT > 1 and DT > T:              # a partial last chunk is handled in the kernels
         DT //= 2
     # staging depth: as many timesteps as fit in LDS (inputs + per-row results), at most DT
     cls = part_input_classes(part)
@@ -228,8 +228,8 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
         if override:
             import dataclasses
             tile = dataclasses.replace(tile, **{k: int(v) for k, v in (kv.split('=') for kv in override.split(','))})
-    assert T % tile.DT == 0 and tile.DT % tile.TS == 0
-    nchunks = T // tile.DT
+    assert tile.DT % tile.TS == 0
+    nchunks = -(-T // tile.DT)
     plan = Plan(B, T, H, M, N, part, cls, [i.dtype for i in inputs], bcast,
                 [s.dtype for s in state], [o.dtype for o in output_t], tile, nchunks)
 

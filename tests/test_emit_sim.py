@@ -29,6 +29,12 @@ RUNS = [
     ('hgrn', '2,8,1,64,1', 'f32', 1),               # vector state (N = 1)
     ('rwkv4', '2,8,1,32,1', 'f32', 0),              # three states, comparisons
     ('mlstm_gates', '2,8,2,16,1', 'f32', 1),        # three outputs
+    # sequence lengths that are not a multiple of the chunk (partial last chunk), and T = 1
+    ('cfg:rwkv7', '1,37,2,128,128', 'f32', 0),
+    ('cfg:mamba1', '2,13,2,128,16', 'f32', 1),
+    ('cfg:mamba2', '2,21,2,64,128', 'bf16', 0),
+    ('rwkv4', '2,11,1,32,1', 'f32', 0),
+    ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1),
 ]
 
 

@@ -172,3 +172,22 @@ def test_other_recurrences(name, dims):
     got = list(res) + [th.zeros_like(p) if t is None else t for t, p in zip(grads, xg + sg)]
     errs = [recurrence.rel_err(a, b) for a, b in zip(got, want)]
     assert max(errs) < 1e-4, errs
+
+
+@pytest.mark.parametrize('name,dims', [('rwkv7', (2, 77, 2, 128, 128)), ('mamba1', (2, 45, 4, 128, 16)),
+                                       ('gated_delta_rule', (2, 1, 2, 128, 128)), ('mamba2', (2, 19, 4, 64, 128))])
+def test_sequence_length_not_a_multiple_of_the_chunk(name, dims):
+    """The reference requires T % chunk == 0 (twopass.py:173); here the last chunk may be
+    partial, down to a single decode step (T = 1)."""
+    print(f'case tail {name} {dims}', flush=True)
+    wl = configs.make(name, dims=dims, dtype=th.float32)
+    dy, dS = configs.upstream_grads(wl)
+    want = recurrence.loop_with_grads(wl.step, wl.inputs, wl.states, dy, dS, dtype=th.float64)
+    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    f = flex_rnn_amd.jit(wl.step)
+    xg = [x.requires_grad_() for x in _gpu(wl.inputs)]
+    sg = [s.requires_grad_() for s in _gpu(wl.states)]
+    res = f(*xg, *sg)
+    grads = th.autograd.grad(res, xg + sg, grad_outputs=[g.cuda() for g in dy + dS])
+    errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
+    assert max(errs) < 1e-4, errs
