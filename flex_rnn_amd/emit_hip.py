@@ -24,12 +24,12 @@ cache key, which is a hash of the source).
 from __future__ import annotations
 
 import math
-from dataclasses import dataclass, field
-from typing import Dict, List, Sequence, Tuple
+from dataclasses import dataclass
+from typing import List, Sequence, Tuple
 
 import torch as th
 
-from .ir import Graph, Node
+from .ir import Graph
 
 DT_CODE = {th.float32: 0, th.bfloat16: 1, th.float16: 2, th.float64: 3}
 
@@ -300,8 +300,8 @@ class Emitter:
         self.tile = plan.tile
         p = self.p
         self.cls = plan.in_cls
-        self.tdep = [not b[1] and plan.T > 1 for b in plan.in_bcast]      # varies with time
-        # an input with T == 1 overall is handled as time-dependent with a single step
+        # staged per timestep: everything but matrix inputs and inputs with a size-1 time axis
+        # (when T == 1 every non-matrix input counts as time-dependent, with a single step)
         self.tdep = [(plan.T == 1 or not b[1]) and c != 'mat' for b, c in zip(plan.in_bcast, self.cls)]
         self.atomic = set(plan.atomic)
         self.jext = p.joint.ext_table()
@@ -324,12 +324,11 @@ class Emitter:
         return ' + '.join(terms)
 
     # ------------------------------------------------------------------ row kernels
-    def _row_kernel_common(self, A: _Args, used_inputs: List[int], R: int, W: int):
+    def _row_kernel_common(self, R: int, W: int):
         """Declarations shared by fw and bw1: thread mapping and staging buffers."""
         t = self.tile
         L, C, G = t.L, t.C, t.G
         MT = W * G * R
-        N = self.plan.N
         src = []
         src.append(f'''  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l = lane % {L}, grp = lane / {L};
@@ -397,7 +396,7 @@ class Emitter:
         out_exts = [(st_ext[0][0], False)] * nout + st_ext + [(st_ext[0][0], False)] * naux
         fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>')
         used_in = [i for i in range(nin) if p.in_names[i] in used]
-        src, MT = self._row_kernel_common(A, used_in, R, W)
+        src, MT = self._row_kernel_common(R, W)
         body = []
         # staging buffers
         tail = plan.T % TS != 0
@@ -520,7 +519,7 @@ class Emitter:
         used_in = [i for i in range(nin) if p.in_names[i] in used_all]
         used_aux = [k for k in range(naux) if p.aux[k] in used_all]
         used_dout = [k for k in range(nout) if p.dout_names[k] in used_all]
-        src, MT = self._row_kernel_common(A, used_in, R, W)
+        src, MT = self._row_kernel_common(R, W)
         body = []
         tail = plan.T % TS != 0
         stg = _Stager(TS, NT, tail)

@@ -20,8 +20,8 @@ tensors instead of from printed code, and carries true broadcast extents.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
-from typing import Dict, Iterable, List, Optional, Sequence, Tuple, Union
+from dataclasses import dataclass
+from typing import Dict, Iterable, List, Sequence, Tuple, Union
 
 Arg = Union[str, float, int, bool]
 

@@ -25,10 +25,10 @@ and saved when `drow` needs them.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Sequence, Tuple
 
-from .ir import Graph, Node
+from .ir import Graph
 
 
 class PartitionError(AssertionError):

@@ -14,10 +14,9 @@ The kernels, their tiling and the layout of the hidden buffers (`state_store`,
 """
 from __future__ import annotations
 
-import hashlib
 import os
-from dataclasses import dataclass, field
-from typing import Callable, Dict, List, Optional, Sequence, Tuple
+from dataclasses import dataclass
+from typing import Callable, List, Optional, Tuple
 
 import torch as th
 
@@ -145,8 +144,7 @@ def classify(inputs, state):
 
 def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
-    assert _is_pow2(N), f'state width N={N} must be a power of two'
-    assert _is_pow2(M), f'state height M={M} must be a power of two'
+    assert _is_pow2(N), f'state width N={N} must be a power of two (the state height M may be any size)'
     # columns per lane: up to 8, so that a row of up to 128 columns fits one 16-lane DPP row
     C = min(N, 8)
     L = N // C

@@ -9,9 +9,8 @@ from __future__ import annotations
 import ctypes
 import hashlib
 import os
-import struct
 import subprocess
-from typing import Optional, Sequence, Tuple
+from typing import Sequence
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)

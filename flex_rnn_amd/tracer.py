@@ -15,7 +15,7 @@ aliasing `_to_copy`).
 """
 from __future__ import annotations
 
-from typing import Callable, Dict, List, Optional, Sequence, Tuple
+from typing import Callable, Dict, List, Sequence, Tuple
 
 import torch
 
@@ -282,6 +282,4 @@ def fx_to_graph(gm: torch.fx.GraphModule, name: str = 'joint') -> Graph:
 
 def trace_step(step: Callable, metas: Sequence[torch.Tensor]) -> Tuple[Graph, int]:
     gm, nfw = trace_joint_fx(step, metas)
-    g = fx_to_graph(gm)
-    # extents of placeholders come from the meta shapes, which is what the caller classified on
-    return g, nfw
+    return fx_to_graph(gm), nfw

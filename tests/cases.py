@@ -22,6 +22,20 @@ CASES = {
     'mlstm_norm': (ops.mlstm_norm, [('row', 'BTH'), ('row', 'BTH'), ('scalar', 'BTH'), ('scalar', 'BTH')], 1),
     'mlstm_cell': (ops.mlstm_cell, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('scalar', 'BTH'), ('scalar', 'BTH'), ('col', 'BTH')], 1),
 }
+
+
+def _zoo(x, g, c, S):
+    """Exercises the emitter's op table: sigmoid, tanh, softplus, where, relu, abs, sqrt, rsqrt, log,
+    reciprocal, maximum/minimum, comparisons, pow, division."""
+    gate = th.sigmoid(g) * th.tanh(x) + F.softplus(x) * 0.1
+    S = S * th.sigmoid(g) + c * th.where(x > 0, gate, 0.2 * gate) + F.relu(x) * 0.05
+    S = S + th.minimum(th.maximum(c, -c), th.ones_like(c)) * th.sqrt(x.abs() + 1.0) / (1.0 + x ** 2)
+    y = (S * th.rsqrt(1.0 + x * x)).sum(-1, True) + th.log(1.0 + c * c) - (1.0 / (2.0 + g.abs())).sum(-1, True)
+    return y, S
+
+
+CASES['zoo'] = (_zoo, [('row', 'BTH'), ('row', 'BT'), ('col', 'BTH')], 1)
+
 # vector-state recurrences (N == 1)
 VECTOR_CASES = {
     'hgrn': (ops.hgrn, [('col', 'BT'), ('col', 'BT')], 1),

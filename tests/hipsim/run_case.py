@@ -23,7 +23,16 @@ def main():
     name, dims, dt, end = sys.argv[1], tuple(int(v) for v in sys.argv[2].split(',')), sys.argv[3], int(sys.argv[4])
     dtype = {'f32': th.float32, 'bf16': th.bfloat16, 'f16': th.float16, 'f64': th.float64}[dt]
     tol = float(sys.argv[5]) if len(sys.argv) > 5 else {'f32': 2e-5, 'f64': 2e-5, 'bf16': 1e-2, 'f16': 3e-3}[dt]
-    if name.startswith('cfg:'):
+    if name.startswith('pattern:'):
+        # gated linear attention with a per-step scalar gain; inputs q, k, v, g, c with the given spans
+        def step(q, k, v, g, c, S):
+            S = S * th.sigmoid(g) + c * (v * k)
+            return (S * q).sum(-1, True), S
+        spec = [tuple(p.split(':')) for p in name[len('pattern:'):].split(',')]
+        table = {'pat': (step, [(c, sp) for c, sp in spec], 1)}
+        step, xs, ss = cases.make_inputs('pat', *dims, dtype=dtype, table=table)
+        ss = [th.randn(dims[0], dims[2], dims[3], dims[4], generator=th.Generator().manual_seed(3)).to(dtype) * 0.3]
+    elif name.startswith('cfg:'):
         wl = configs.make(name[4:], dims=dims, dtype=dtype)
         step, xs, ss = wl.step, wl.inputs, wl.states
     else:

@@ -35,6 +35,13 @@ RUNS = [
     ('cfg:mamba2', '2,21,2,64,128', 'bf16', 0),
     ('rwkv4', '2,11,1,32,1', 'f32', 0),
     ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1),
+    # the emitter's op table (sigmoid, tanh, softplus, where, relu, sqrt, rsqrt, log, min/max, ...)
+    ('zoo', '2,8,2,16,16', 'f32', 1),
+    # state heights that are not a power of two (row masking), fp64 and fp16 I/O
+    ('cfg:rwkv7', '1,16,1,24,128', 'f32', 0),
+    ('gla', '2,8,2,100,32', 'f32', 1),
+    ('zoo', '1,8,2,5,8', 'f64', 0),
+    ('gla', '1,8,2,16,16', 'f16', 1),
 ]
 
 
@@ -42,3 +49,24 @@ RUNS = [
 def test_emitted_kernels_on_cpu(case, dims, dtype, end):
     r = subprocess.run([sys.executable, RUNNER, case, dims, dtype, str(end)], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
+
+
+def _random_pattern_case(seed):
+    """A gated linear-attention step whose five inputs get random classes-compatible broadcast
+    patterns over (B, T, H); returns the argument string of run_case.py's `pattern:` mode."""
+    import random
+    rnd = random.Random(seed)
+    spans = []
+    for cls in ('row', 'row', 'col', 'row', 'scalar'):
+        sp = ''.join(d for d in 'BTH' if rnd.random() < 0.7)
+        spans.append(f'{cls}:{sp}')
+    # at least one input must span each of B, T, H (the state fixes B and H; T comes from the inputs)
+    spans[0] = 'row:BTH'
+    return 'pattern:' + ','.join(spans)
+
+
+@pytest.mark.parametrize('seed', range(6))
+def test_random_broadcast_patterns(seed):
+    case = _random_pattern_case(seed)
+    r = subprocess.run([sys.executable, RUNNER, case, '2,8,3,8,16', 'f32', str(seed % 2)], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, f'{case}\nrc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'

@@ -156,7 +156,8 @@ def test_check_grad_and_benchmark_helpers():
 
 @pytest.mark.parametrize('name,dims', [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn', (2, 32, 2, 32, 16)),
                                        ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
-                                       ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32))])
+                                       ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)),
+                                       ('zoo', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32))])
 def test_other_recurrences(name, dims):
     print(f'case {name} {dims}', flush=True)
     step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)
@@ -191,3 +192,22 @@ def test_sequence_length_not_a_multiple_of_the_chunk(name, dims):
     grads = th.autograd.grad(res, xg + sg, grad_outputs=[g.cuda() for g in dy + dS])
     errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
     assert max(errs) < 1e-4, errs
+
+
+@pytest.mark.parametrize('dtype,tol', [(th.float16, 3e-3), (th.float64, 1e-4)])
+def test_half_and_double_io(dtype, tol):
+    """fp16 I/O; fp64 I/O is accepted and computed in fp32, as in the reference (to_cuda.py:169)."""
+    print(f'case io dtype {dtype}', flush=True)
+    step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
+    f = flex_rnn_amd.jit(step)
+    xg = [x.requires_grad_() for x in _gpu(xs)]
+    sg = [s.requires_grad_() for s in _gpu(ss)]
+    res = f(*xg, *sg)
+    assert res[0].dtype == dtype and res[1].dtype == dtype
+    g = th.Generator().manual_seed(9)
+    gy = [th.randn(r.shape, generator=g).to(dtype) for r in res]
+    grads = th.autograd.grad(res, xg + sg, [t.cuda() for t in gy])
+    want = recurrence.loop_with_grads(step, xs, ss, gy[:1], gy[1:])
+    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
+    assert max(errs) < tol, errs

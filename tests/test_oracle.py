@@ -1,7 +1,5 @@
 """Pins the CPU oracle (oracle/recurrence.py) with closed forms, brute force and invariants,
 and checks the package's `jit.naive` against it."""
-import math
-
 import pytest
 import torch as th
 

@@ -16,13 +16,18 @@ from flex_rnn_amd.launch import compile_plan  # noqa: E402
 OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn', (2, 32, 2, 32, 16)),
          ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
          ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)), ('gla', (1, 16, 1, 16, 16)),
-         ('gla', (1, 32, 1, 16, 16)), ('delta_rule', (2, 32, 2, 16, 16)), ('gated_delta_rule', (2, 32, 2, 16, 16))]
+         ('gla', (1, 32, 1, 16, 16)), ('delta_rule', (2, 32, 2, 16, 16)), ('gated_delta_rule', (2, 32, 2, 16, 16)),
+         ('zoo', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32))]
 
 
 def warm(force=False, seen=None):
     n = 0
     for name, dims in OTHER:
         step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)
+        plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
+        n += len(compile_plan(plan, force=force, seen=seen))
+    for dtype in (th.float16, th.float64):
+        step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
         n += len(compile_plan(plan, force=force, seen=seen))
     for name in ('rwkv7', 'gated_delta_rule'):
