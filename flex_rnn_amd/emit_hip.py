@@ -254,7 +254,10 @@ class _Stager:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
             if self._linear(ln):
-                out += f'  const i64 pb_{name} = {fn("0", f"(tid % {ln})")};\n  const int tb_{name} = tid / {ln};\n'
+                if self.tail:       # the timestep is clamped per thread, keep it out of the base
+                    out += f'  const i64 pb_{name} = {fn("0", f"(tid % {ln})")};\n  const int tb_{name} = tid / {ln};\n'
+                else:               # base holds the thread's own timestep; loads add a wave-uniform offset
+                    out += f'  const i64 pb_{name} = {fn(f"(tid / {ln})", f"(tid % {ln})")};\n'
         return out
 
     def _loop(self, ln, body, ind):
@@ -269,9 +272,11 @@ class _Stager:
     def load(self, t0: str, ind: str) -> str:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
-            if self._linear(ln):
+            if self._linear(ln) and self.tail:
                 t = self._clamp(f'({t0}) + tb_{name} + it_ * {self.NT // ln}')
                 idx = f'pb_{name} + (i64)({t}) * {ts}'
+            elif self._linear(ln):
+                idx = f'pb_{name} + (i64)(({t0}) + it_ * {self.NT // ln}) * {ts}'
             else:
                 idx = fn(self._clamp(f'({t0}) + tt_'), 'x_')
             out += self._loop(ln, f'pf_{name}[it_] = ldr<{dt}>({ptr}, {idx});', ind)
