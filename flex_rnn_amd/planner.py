@@ -215,7 +215,13 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
     assert all(list(i.shape) == [B, H, M, 1] for i in output_t), [i.shape for i in output_t]
     assert all(i.dtype in SUPPORTED_DTYPES for i in output_t)
 
-    metas = tuple(th.empty(j.shape[-2:], dtype=j.dtype, device='meta') for j in tuple(inputs_t) + tuple(state))
+    # Trace on [m, n] shapes.  With a single state row (M == 1) a [1, n] state would be
+    # indistinguishable from a row-broadcast operand and the graph would lose its row extents;
+    # it is traced with two rows instead (inputs keep their size-1 row axis, i.e. are broadcast
+    # over rows, which is the same thing for one row).
+    Mt = 2 if M == 1 else M
+    metas = tuple(th.empty(j.shape[-2:], dtype=j.dtype, device='meta') for j in inputs_t) \
+        + tuple(th.empty((Mt, N), dtype=s.dtype, device='meta') for s in state)
     joint, nfw = tracer.trace_step(step, metas)
     assert nfw == noutputs + nstates
     part = partition(joint, ninputs, nstates, noutputs, cls)

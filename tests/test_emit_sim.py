@@ -42,6 +42,9 @@ RUNS = [
     ('gla', '2,8,2,100,32', 'f32', 1),
     ('zoo', '1,8,2,5,8', 'f64', 0),
     ('gla', '1,8,2,16,16', 'f16', 1),
+    # a single state row (M = 1), down to a scalar state (M = N = 1)
+    ('mlstm_gates', '2,8,2,1,1', 'f32', 1),
+    ('gla', '2,8,2,1,16', 'f32', 0),
 ]
 
 

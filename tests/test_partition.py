@@ -36,6 +36,11 @@ def test_partition_vector_state(name):
     _check(name, 2, 8, 2, 8, 1, DT=4)
 
 
+@pytest.mark.parametrize('name,M,N', [('mlstm_gates', 1, 1), ('gla', 1, 8), ('delta_rule', 1, 4)])
+def test_partition_single_row_state(name, M, N):
+    _check(name, 2, 8, 2, M, N, DT=4)
+
+
 def test_aux_daux_of_rwkv7():
     plan = _check('rwkv7_decay', 1, 4, 1, 4, 4, DT=2)
     p = plan.part

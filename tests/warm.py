@@ -20,8 +20,38 @@ OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn'
          ('zoo', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32))]
 
 
-def warm(force=False, seen=None):
+EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
+
+
+def warm_examples(force=False, seen=None):
+    """Dry-runs every example layer on meta tensors, captures the plans its jit objects
+    request and compiles their kernels."""
+    import flex_rnn_amd
+    jit_mod = sys.modules['flex_rnn_amd.jit']        # (the package attribute `jit` is the class)
+    from flex_rnn_amd import examples
     n = 0
+    orig = jit_mod.build_twopass
+
+    def capture(step, inputs, state, dryrun=False, tile=None):
+        nonlocal n
+        metas = [t.to('meta') for t in inputs], [t.to('meta') for t in state]
+        plan = planner.make_plan(step, *metas, tile)[0]
+        n += len(compile_plan(plan, force=force, seen=seen))
+        return orig(step, inputs, state, dryrun=True, tile=tile)
+
+    jit_mod.build_twopass = capture
+    try:
+        for op in examples.OPS:
+            a = EXAMPLE_ARGS
+            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta')
+            layer(*inputs)
+    finally:
+        jit_mod.build_twopass = orig
+    return n
+
+
+def warm(force=False, seen=None):
+    n = warm_examples(force, seen)
     for name, dims in OTHER:
         step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
