@@ -211,3 +211,30 @@ def test_half_and_double_io(dtype, tol):
     want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
     errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
     assert max(errs) < tol, errs
+
+
+def test_torch_compile_default_backend_and_side_stream():
+    """The default torch.compile backend (inductor) fuses the pointwise work around the op; and
+    launches follow torch's current stream."""
+    print('case inductor + side stream', flush=True)
+    step, xs, ss = cases.make_inputs('delta_rule', 2, 32, 2, 16, 16, dtype=th.float32)
+    f = flex_rnn_amd.jit(step)
+    xs, ss = _gpu(xs), _gpu(ss)
+
+    def layer(q, k, v, beta, S):
+        y, S = f(th.tanh(q), k, v, th.sigmoid(beta), S)
+        return y * 2.0 + 1.0, S
+
+    def run(fn):
+        args = [x.clone().requires_grad_() for x in xs + ss]
+        out = fn(*args)
+        return list(out) + list(th.autograd.grad(out, args, [th.ones_like(o) for o in out]))
+
+    ref = run(layer)
+    got = run(th.compile(layer, fullgraph=True))
+    assert max(recurrence.rel_err(a, b) for a, b in zip(got, ref)) < 1e-5
+    side = th.cuda.Stream()
+    with th.cuda.stream(side):
+        got = run(layer)
+    side.synchronize()
+    assert all(th.equal(a, b) for a, b in zip(got, ref))
