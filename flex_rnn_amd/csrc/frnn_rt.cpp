@@ -41,7 +41,7 @@ int fail(int code, const char* fmt, ...) {
 // ---------------------------------------------------------------- HIP entry points
 typedef int hipError_t;
 struct HipApi {
-  hipError_t (*ModuleLoad)(void**, const char*) = nullptr;
+  hipError_t (*ModuleLoadData)(void**, const void*) = nullptr;
   hipError_t (*ModuleUnload)(void*) = nullptr;
   hipError_t (*ModuleGetFunction)(void**, void*, const char*) = nullptr;
   hipError_t (*ModuleLaunchKernel)(void*, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned,
@@ -59,7 +59,7 @@ HipApi& hip() {
   static std::once_flag once;
   std::call_once(once, [] {
     void* h = RTLD_DEFAULT;
-    if (!dlsym(RTLD_DEFAULT, "hipModuleLoad")) {
+    if (!dlsym(RTLD_DEFAULT, "hipModuleLoadData")) {
       h = dlopen("libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
       if (!h) h = dlopen("libamdhip64.so.7", RTLD_NOW | RTLD_GLOBAL);
       if (!h) h = dlopen("/opt/rocm/lib/libamdhip64.so", RTLD_NOW | RTLD_GLOBAL);
@@ -71,7 +71,7 @@ HipApi& hip() {
 #define FRNN_SYM(field, name)                                              \
   *(void**)(&api.field) = dlsym(h, name);                                  \
   if (!api.field) { api.why = std::string("missing HIP symbol ") + name; return; }
-    FRNN_SYM(ModuleLoad, "hipModuleLoad")
+    FRNN_SYM(ModuleLoadData, "hipModuleLoadData")
     FRNN_SYM(ModuleUnload, "hipModuleUnload")
     FRNN_SYM(ModuleGetFunction, "hipModuleGetFunction")
     FRNN_SYM(ModuleLaunchKernel, "hipModuleLaunchKernel")
@@ -159,6 +159,7 @@ std::vector<std::string> split_ws(const char* s) {
 
 struct frnn_module_s {
   void* mod;
+  std::vector<char> image;   // the code object bytes; kept for the lifetime of the module
 };
 
 extern "C" {
@@ -242,10 +243,34 @@ int frnn_module_load(const char* path, frnn_module_t* out) {
   if (!path || !out) return fail(FRNN_ERR_ARG, "frnn_module_load: null argument");
   HipApi& h = hip();
   if (!h.ok) return fail(FRNN_ERR_NO_HIP, "%s", h.why.c_str());
-  void* mod = nullptr;
-  hipError_t e = h.ModuleLoad(&mod, path);
-  if (e != 0) return hip_fail("hipModuleLoad", e);
-  *out = new frnn_module_s{mod};
+  // The image is read here and handed over in memory: the file may be replaced by a rebuild
+  // later, and the module must not depend on it.
+  FILE* f = fopen(path, "rb");
+  if (!f) return fail(FRNN_ERR_IO, "cannot open code object %s: %s", path, strerror(errno));
+  fseek(f, 0, SEEK_END);
+  long n = ftell(f);
+  fseek(f, 0, SEEK_SET);
+  frnn_module_s* m = new frnn_module_s{nullptr, std::vector<char>((size_t)(n > 0 ? n : 0))};
+  size_t got = n > 0 ? fread(m->image.data(), 1, (size_t)n, f) : 0;
+  fclose(f);
+  if (n <= 0 || got != (size_t)n) {
+    delete m;
+    return fail(FRNN_ERR_IO, "cannot read code object %s", path);
+  }
+  // refuse anything that is not an offload bundle or an ELF image before the driver parses it
+  static const char kBundle[] = "__CLANG_OFFLOAD_BUNDLE__";
+  bool bundle = (size_t)n > sizeof kBundle && memcmp(m->image.data(), kBundle, sizeof kBundle - 1) == 0;
+  bool elf = n > 64 && memcmp(m->image.data(), "\177ELF", 4) == 0;
+  if (!bundle && !elf) {
+    delete m;
+    return fail(FRNN_ERR_IO, "%s is not a code object (damaged cache entry?)", path);
+  }
+  hipError_t e = h.ModuleLoadData(&m->mod, m->image.data());
+  if (e != 0) {
+    delete m;
+    return hip_fail("hipModuleLoadData", e);
+  }
+  *out = m;
   return FRNN_OK;
 }
 

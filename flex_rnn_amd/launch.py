@@ -53,9 +53,18 @@ class CompiledPlan:
         self.kernels = {}
         self.modules = []
         for spec, path in built:
-            mod = runtime.Module(path)
+            try:
+                mod = runtime.Module(path)
+                kern = mod.kernel(spec.name)
+            except runtime.RuntimeError_ as first:
+                if 'no HIP runtime' in str(first) or 'no ROCm-capable device' in str(first).lower():
+                    raise
+                # a truncated / corrupt cache entry: rebuild it once, then give up loudly
+                path = runtime.compile_kernel(spec.name, spec.source, force=True)
+                mod = runtime.Module(path)
+                kern = mod.kernel(spec.name)
             self.modules.append(mod)
-            self.kernels[spec.name] = (spec, mod.kernel(spec.name))
+            self.kernels[spec.name] = (spec, kern)
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):

@@ -53,7 +53,9 @@ const char* frnn_last_error(void);
 int frnn_compile(const char* src, size_t len, const char* arch, const char* opts,
                  const char* cache_dir, const char* key, char* out_path, size_t cap);
 
-/* Load a code object file into the current device's context.
+/* Load a code object file into the current device's context.  The file is read into memory
+ * owned by the module (hipModuleLoadData), so it may be rebuilt or removed afterwards; a file
+ * that is neither an offload bundle nor an ELF image is rejected with FRNN_ERR_IO.
  * Replaces: the dlopen done by cpp_extension.load (to_cuda.py:279). */
 int frnn_module_load(const char* path, frnn_module_t* out);
 

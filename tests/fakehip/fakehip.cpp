@@ -3,7 +3,7 @@
 #include <stddef.h>
 extern "C" {
 int g_extra_ok = 0; unsigned char g_args[8192]; size_t g_nargs = 0; unsigned g_dims[7]; void* g_stream; void* g_kparams;
-int hipModuleLoad(void** m, const char* p) { *m = (void*)0x1111; return 0; }
+int hipModuleLoadData(void** m, const void* image) { *m = (void*)0x1111; return 0; }
 int hipModuleUnload(void* m) { return 0; }
 int hipModuleGetFunction(void** f, void* m, const char* n) { *f = (void*)0x2222; return 0; }
 int hipModuleLaunchKernel(void* f, unsigned gx, unsigned gy, unsigned gz, unsigned bx, unsigned by, unsigned bz, unsigned sh, void* stream, void** kp, void** extra) {

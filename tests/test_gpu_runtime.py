@@ -80,3 +80,26 @@ def test_probe_launch():
 
 def test_device_cus():
     assert runtime.device_cus() > 0
+
+
+def test_corrupt_cache_entry_is_rebuilt(tmp_path, monkeypatch):
+    """A damaged code object in the cache is recompiled on load instead of failing for good."""
+    import glob
+    import os
+
+    import flex_rnn_amd
+    from flex_rnn_amd import ops
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    g = th.Generator().manual_seed(0)
+    q, k = [th.randn(1, 16, 1, 1, 16, generator=g).cuda() for _ in range(2)]
+    v = th.randn(1, 16, 1, 16, 1, generator=g).cuda()
+    gate = -th.rand(1, 16, 1, 1, 16, generator=g).cuda()
+    S = th.zeros(1, 1, 16, 16).cuda()
+    y0, _ = flex_rnn_amd.jit(ops.gla)(q, k, v, gate, S)          # fills the cache
+    files = glob.glob(os.path.join(str(tmp_path), 'frnn_fw_*.hsaco'))
+    assert len(files) == 1
+    with open(files[0], 'wb') as f:
+        f.write(b'not a code object')
+    y1, _ = flex_rnn_amd.jit(ops.gla)(q, k, v, gate, S)          # new instance: loads from the cache
+    th.cuda.synchronize()
+    assert th.equal(y0, y1) and os.path.getsize(files[0]) > 1000

@@ -73,7 +73,7 @@ def test_launch_marshalling_against_stand_in_hip(runtime_lib, tmp_path):
         fake = ctypes.CDLL({str(so)!r}, mode=ctypes.RTLD_GLOBAL)
         from flex_rnn_amd import runtime
         assert runtime.device_cus() == 256
-        m = runtime.Module('/nonexistent'); k = m.kernel('x')
+        open({str(so)!r} + '.img', 'wb').write(bytes([127]) + b'ELF' + bytes(100)); m = runtime.Module({str(so)!r} + '.img'); k = m.kernel('x')
         buf = struct.pack('<q5q', 0x7f0012345678, 1, 2, 3, 4, 5) + struct.pack('<5q', 7, 8, 9, 10, 11)
         k.launch((2, 3, 4), (64, 1, 1), buf, stream=0xabc)
         n = ctypes.c_size_t.in_dll(fake, 'g_nargs').value
@@ -89,6 +89,13 @@ def test_launch_marshalling_against_stand_in_hip(runtime_lib, tmp_path):
                 assert 'frnn_launch' in str(e), e
             else:
                 raise SystemExit('accepted ' + str(bad))
+        open({str(so)!r} + '.bad', 'wb').write(b'not a code object')
+        try:
+            runtime.Module({str(so)!r} + '.bad')
+        except RuntimeError as e:
+            assert 'not a code object' in str(e), e
+        else:
+            raise SystemExit('loaded garbage')
         print('ok')
     ''')
     r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
