@@ -145,32 +145,43 @@ def classify(inputs, state):
 def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
     assert _is_pow2(N), f'state width N={N} must be a power of two (the state height M may be any size)'
-    # columns per lane: up to 8, so that a row of up to 128 columns fits one 16-lane DPP row
-    C = min(N, 8)
-    L = N // C
-    while L > 64:
-        C *= 2
-        L = N // C
-    G = 64 // L
     nst = part.nstates + len(part.mat_idx)
-    # rows per lane: bounded by the register budget (state + new state + temporaries) ...
-    R = _pow2_floor(max(1, min(64 // max(C * nst, 1), 8)))
-    while R > 1 and G * R > M:          # ... and by the rows that exist
-        R //= 2
 
-    def waves_per_wg(R_):
-        return max(1, min(4, M // (G * R_))) if G * R_ <= M else 1
+    def geometry(C_):
+        L_ = N // C_
+        G_ = 64 // L_
+        # rows per lane: bounded by the register budget (state + new state + temporaries) ...
+        R_ = _pow2_floor(max(1, min(64 // max(C_ * nst, 1), 8)))
+        while R_ > 1 and G_ * R_ > M:          # ... by the rows that exist ...
+            R_ //= 2
 
-    def total_waves(R_):
-        W_ = waves_per_wg(R_)
-        return B * H * max(1, -(-M // (W_ * G * R_))) * W_
+        def waves_per_wg(r):
+            return max(1, min(4, M // (G_ * r))) if G_ * r <= M else 1
 
-    # ... and small enough that every SIMD holds at least two waves (latency hiding)
-    while R > 1 and total_waves(R) < 2 * 4 * n_cu:
-        R //= 2
-    W = waves_per_wg(R)
+        def total_waves(r):
+            w = waves_per_wg(r)
+            return B * H * max(1, -(-M // (w * G_ * r))) * w
+
+        # ... and small enough that every SIMD holds at least two waves (latency hiding)
+        while R_ > 1 and total_waves(R_) < 2 * 4 * n_cu:
+            R_ //= 2
+        return L_, G_, R_, waves_per_wg(R_), total_waves(R_)
+
+    # columns per lane: up to 8, so that a row of up to 128 columns fits one 16-lane DPP row;
+    # fewer when the whole problem would otherwise give the chip too few waves (narrow states)
+    C = min(N, 8)
+    while N // C > 64:
+        C *= 2
+    L, G, R, W, waves = geometry(C)
+    while C > 2 and N // (C // 2) <= 64 and waves < 2 * 4 * n_cu:
+        C //= 2
+        L, G, R, W, waves = geometry(C)
     MT = W * G * R
-    DT = 8 if part.dstep_needs_state else 16
+    if part.dstep_needs_state:
+        # the reverse scan keeps the DT recomputed states of a chunk in registers
+        DT = max(2, min(16, _pow2_floor(128 // max(R * C * nst, 1))))
+    else:
+        DT = 16
     while DT > 1 and DT > T:              # a partial last chunk is handled in the kernels
         DT //= 2
     # staging depth: as many timesteps as fit in LDS (inputs + per-row results), at most DT
