@@ -80,6 +80,16 @@ def main():
     wall = time.perf_counter() - t0
     ev = compiled.profile_events
     compiled.profile_events = None
+    # forward only (outside the headline region): same inputs, no autograd
+    with th.no_grad():
+        for _ in range(2):
+            f(*xs, *ss)
+        th.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            f(*xs, *ss)
+        th.cuda.synchronize()
+        fwd_ms = (time.perf_counter() - t1) * 1e3 / args.steps
     ms_per_step = wall * 1e3 / args.steps
     tokens = B * T
     value = tokens / (wall / args.steps)
@@ -128,6 +138,9 @@ def main():
         'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
         'roofline': roofline, 'cpu_baseline': cpu,
         'gpu_kernel_ms_per_step': round(gpu_ms, 4),
+        'forward_only': {'ms_per_step': round(fwd_ms, 4), 'tokens_per_s': round(tokens / (fwd_ms * 1e-3), 1),
+                         'achieved_TFLOPs': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12, 3),
+                         'frac': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4)},
     }
     print(json.dumps(out))
 
