@@ -712,6 +712,9 @@ class Emitter:
         IPB = max(1, 64 // N)
         NT = max(64, N)
         HB = max(1, getattr(t, 'HB', 1))
+        MS = max(1, getattr(t, 'MS', 1))
+        MR = -(-plan.M // MS)               # rows per instance
+        PD = 4                              # checkpoint rows in flight ahead of the row loop
         assert plan.H % HB == 0
         A = _Args()
         nin, nst, nout = p.ninputs, p.nstates, p.noutputs
@@ -750,6 +753,9 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
 }}
 '''
         b = []
+        rows_decl = ('  const int mlo = 0, mhi = M;' if MS == 1 else
+                     f'  const int mlo = blockIdx.z * {MR}, mhi = min(M, mlo + {MR});   // rows of this instance\n'
+                     '  if (mlo >= M) return;')
         b.append(f'''  const int tid = threadIdx.x;
   const int n = tid % {N};
   const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
@@ -761,6 +767,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   const int HG = H / {HB};                     // head groups; an instance walks {HB} heads
   const int b = blockIdx.y / HG, h0 = (blockIdx.y % HG) * {HB};
   const int t0 = ch * {DT};
+{rows_decl}
   const int nt = {f"min({DT}, T - t0)" if self.tail_dt else DT};          // timesteps of this chunk
   (void)nt;
 ''')
@@ -838,7 +845,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                             f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
                 rowops.append((f's_dy{k}', ldy, f'dy{k}'))
         MB = 1
-        while MB * 2 <= plan.M and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
+        while MB * 2 <= MR and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
             MB *= 2
         lanes = min(N, NT)          # lanes of one instance
         for nm_lds, _, _ in rowops:
@@ -848,23 +855,32 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for k in range(nst):
             b.append(f'  const float* sckp{k} = (const float*){A.p(f"sck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
             b.append(f'  const float* dckp{k} = (const float*){A.p(f"dck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
-            b.append(f'  float Snx{k} = sckp{k}[0];\n  float Dnx{k} = dckp{k}[0];\n')
-        b.append(f'  for (int m0 = 0; m0 < M; m0 += {MB}) {{\n')
+            for j in range(PD):
+                b.append(f'  float Sq{k}_{j} = sckp{k}[min(mlo + {j}, M - 1) * {N}];\n  float Dq{k}_{j} = dckp{k}[min(mlo + {j}, M - 1) * {N}];\n')
+        b.append(f'  for (int m0 = mlo; m0 < mhi; m0 += {MB}) {{\n')
         if rowops:
             b.append('    __syncthreads();\n')
-            b.append(f'    for (int e_ = n; e_ < {MB * DT}; e_ += {lanes}) {{ const int tt_ = e_ / {MB}, mm_ = e_ % {MB}; '
-                     f'const int mc_ = min(m0 + mm_, M - 1);\n')
+            # fixed trip count, fully unrolled: every load of the block is in flight before the
+            # first LDS write waits for one
+            trips = -(-(MB * DT) // lanes)
+            guard = '' if (MB * DT) % lanes == 0 else f'if (e_ < {MB * DT}) '
+            b.append(f'#pragma unroll {min(trips, 2)}\n    for (int i_ = 0; i_ < {trips}; i_++) {{ const int e_ = n + i_ * {lanes}; {guard}{{ '
+                     f'const int tt_ = e_ / {MB}, mm_ = e_ % {MB}; const int mc_ = min(m0 + mm_, M - 1);\n')
             for nm_lds, ld, _ in rowops:
                 b.append(f'      {nm_lds}[inst][mm_][tt_] = {ld("tt_", "mc_")};\n')
-            b.append('    }\n    __syncthreads();\n')
-        b.append(f'  for (int mm = 0; mm < {MB}; mm++) {{\n    const int m = m0 + mm;\n    if (m >= M) break;\n')
+            b.append('    } }\n    __syncthreads();\n')
+        b.append(f'#pragma unroll {min(PD, MB)}\n  for (int mm = 0; mm < {MB}; mm++) {{\n    const int m = m0 + mm;\n    if (m >= mhi) break;\n')
         for k in range(nst):
-            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Snx{k};\n')
-            b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dnx{k};\n')
-        b.append('    { const int mn_ = min(m + 1, M - 1);\n')
+            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Sq{k}_0;\n')
+            b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dq{k}_0;\n')
+        # checkpoint rows are fetched PD rows ahead of their use: one row of arithmetic is shorter
+        # than a trip to HBM
+        b.append(f'    {{ const int mn_ = min(m + {PD}, M - 1);\n')
         for k in range(nst):
-            b.append(f'      Snx{k} = sckp{k}[mn_ * {N}];\n')
-            b.append(f'      Dnx{k} = dckp{k}[mn_ * {N}];\n')
+            for j in range(PD - 1):
+                b.append(f'      Sq{k}_{j} = Sq{k}_{j + 1}; Dq{k}_{j} = Dq{k}_{j + 1};\n')
+            b.append(f'      Sq{k}_{PD - 1} = sckp{k}[mn_ * {N}];\n')
+            b.append(f'      Dq{k}_{PD - 1} = dckp{k}[mn_ * {N}];\n')
         b.append('    }\n')
         for nm_lds, _, pref in rowops:
             for tt in range(DT):
@@ -943,7 +959,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             if tail and not bT:
                 cond += f' && t0 + {tt} < T'
             idx = out_index(i, tt, hexpr)
-            if bB or bT or (bH and HB < plan.H):
+            if bB or bT or (bH and HB < plan.H) or MS > 1:
                 return f'{ind}if ({cond}) atomic_addf({A.p(nmv)}, {idx}, {val});\n'
             dt = 0 if i in self.atomic else DT_CODE[plan.in_dtypes[i]]      # broadcast inputs use fp32 scratch
             return f'{ind}if ({cond}) stf<{dt}>({A.p(nmv)}, {idx}, {val});\n'
@@ -951,12 +967,31 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         tacc = [i for i in rs if bflags(i)[1]]
         for i in tacc:
             b.append(f'  float gt{i} = 0.0f;\n')
+        # sums over rows and columns: the column part is a reduction over the instance's lanes.
+        # With more than one wave per instance all of them share one pair of barriers.
+        nred = [j for j, mname in enumerate(p.msums)
+                if 1 in nm_[mname].dims and self.jext[nm_[mname].args[0]][1]]
+        batched = N > 64 and bool(nred)
+        if batched:
+            NW = N // 64
+            b.append(f'  __shared__ float red_ms[{len(nred) * DT}][{NW}];\n')
+            for q, j in enumerate(nred):
+                for tt in range(DT):
+                    b.append(f'  acc{j}_{tt} = grp_allreduce<64>(acc{j}_{tt});\n')
+            b.append('  __syncthreads();\n  if ((tid & 63) == 0) {\n')
+            for q, j in enumerate(nred):
+                for tt in range(DT):
+                    b.append(f'    red_ms[{q * DT + tt}][tid >> 6] = acc{j}_{tt};\n')
+            b.append('  }\n  __syncthreads();\n')
+            for q, j in enumerate(nred):
+                for tt in range(DT):
+                    b.append(f'  acc{j}_{tt} = ' + ' + '.join(f'red_ms[{q * DT + tt}][{w}]' for w in range(NW)) + ';\n')
         for tt in range(DT):
             b.append('  {\n')
             for j, mname in enumerate(p.msums):
                 node = nm_[mname]
                 opext = self.jext[node.args[0]]
-                if 1 in node.dims and opext[1]:
+                if 1 in node.dims and opext[1] and not batched:
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}(acc{j}_{tt});\n')
                 else:
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = acc{j}_{tt};\n')
@@ -987,4 +1022,4 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     b.append(write_out(i, tt, 'h0', f'gh{i}_{tt}', '  '))
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
         source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + kernel
-        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})', '1'))
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})', str(MS)))

@@ -64,6 +64,8 @@ class Partition:
     epi: Graph = None
     dstep_needs_state: bool = False
     mat_in_dstep: bool = False       # matrix-input grads are accumulated by the reverse scan (it has the state)
+    epi_linear: bool = False         # `epi` is linear and homogeneous in the msums: partial row sums may be
+                                     # mapped separately and the results added
 
     def describe(self) -> str:
         return '\n\n'.join(g.code() for g in (self.fw, self.restep, self.dstep, self.drow, self.epi))
@@ -74,6 +76,37 @@ def _depends(graph: Graph, seeds: Sequence[str]) -> Dict[str, bool]:
     for n in graph.nodes:
         dep[n.name] = any(dep[a] for a in n.value_args())
     return dep
+
+
+def _linear_in(graph: Graph, seeds: Sequence[str]) -> bool:
+    """True if every output of `graph` is a linear homogeneous function of the inputs named in
+    `seeds` (their coefficients may depend on the other inputs in any way)."""
+    IND, LIN, NON = 0, 1, 2          # independent of the seeds / linear in them / anything else
+    kind = {i: (LIN if i in seeds else IND) for i in graph.inputs}
+
+    def k(a):
+        return kind[a] if isinstance(a, str) else IND
+
+    for n in graph.nodes:
+        ks = [k(a) for a in n.args]
+        if all(x == IND for x in ks):
+            r = IND
+        elif NON in ks:
+            r = NON
+        elif n.op in ('neg', 'copy', 'sum'):
+            r = ks[0]
+        elif n.op in ('add', 'sub'):
+            r = LIN if ks == [LIN, LIN] else NON
+        elif n.op == 'mul':
+            r = LIN if sorted(ks) == [IND, LIN] else NON
+        elif n.op == 'div':
+            r = LIN if ks == [LIN, IND] else NON
+        elif n.op == 'where':
+            r = LIN if ks == [IND, LIN, LIN] else NON
+        else:
+            r = NON
+        kind[n.name] = r
+    return all(kind[o] == LIN for o in graph.outputs)
 
 
 def classify_index(ext: Tuple[bool, bool]) -> str:
@@ -202,5 +235,6 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
                   out_names, nst_names, din_names, dst_names, aux, daux, msums,
                   col_idx, row_idx, scalar_idx, mat_idx,
                   fw=fw, restep=restep, dstep=dstep, drow=drow, epi=epi,
-                  dstep_needs_state=dstep_needs_state, mat_in_dstep=mat_in_dstep)
+                  dstep_needs_state=dstep_needs_state, mat_in_dstep=mat_in_dstep,
+                  epi_linear=_linear_in(epi, set(msums)))
     return p

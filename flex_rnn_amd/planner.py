@@ -80,6 +80,8 @@ class TileConfig:
     R1: int = 0          # rows per lane / waves in bw1 (0 = same as fw)
     W1: int = 0
     HB: int = 1          # heads walked by one gradient-kernel instance (sums head-broadcast grads in registers)
+    MS: int = 1          # instances sharing the rows of one (batch, head, chunk) in the gradient kernel;
+                         # above 1 the row/scalar-input grads are summed across them with atomics
 
     @property
     def G(self): return 64 // self.L
@@ -105,7 +107,8 @@ class Plan:
 
     @property
     def atomic(self) -> List[int]:
-        return [i for i, b in enumerate(self.in_bcast) if any(b)]
+        split = set(self.part.row_idx + self.part.scalar_idx) if self.tile.MS > 1 else set()
+        return [i for i, b in enumerate(self.in_bcast) if any(b) or i in split]
 
 
 def classify(inputs, state):
@@ -194,16 +197,18 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
         TS //= 2
     if part.dstep_needs_state:
         TS = DT
-    # gradient kernel: walk several heads per instance when a row/scalar input is shared by all
-    # heads (its gradient then needs no atomics inside the group), keeping >= 2 waves per SIMD
-    HB = 1
-    if in_bcast is not None and any(in_bcast[i][2] for i in part.row_idx + part.scalar_idx):
-        ipb = max(1, 64 // N)
-        waves = lambda hb: B * (H // hb) * -(-(T // DT) // ipb) * max(1, N // 64)
-        HB = H & -H                     # largest power of two dividing H
-        while HB > 1 and waves(HB) < 2 * 4 * n_cu:
-            HB //= 2
-    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, HB=HB)
+    # gradient kernel: one instance per (batch, head, chunk) walks all M rows.  When that gives the
+    # chip too few waves (narrow states pack several instances into a wave), the rows are split
+    # over MS instances whose row/scalar-input grads meet in fp32 atomics; needs an epilogue that
+    # is linear in the row sums.  Walking several heads per instance (HB > 1) saves atomics on
+    # head-shared inputs but costs registers and parallelism; measured slower, so it stays 1.
+    ipb = max(1, 64 // N)
+    waves2 = B * H * -(-(-(-T // DT)) // ipb) * max(1, N // 64)
+    MS = 1
+    if part.epi_linear:
+        while waves2 * MS < 32 * 4 * n_cu and -(-M // (2 * MS)) >= 8:
+            MS *= 2
+    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, HB=1, MS=MS)
 
 
 def part_input_classes(part: Partition) -> List[str]:

@@ -54,6 +54,25 @@ def test_emitted_kernels_on_cpu(case, dims, dtype, end):
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
 
 
+# explicit tile overrides: gradient-kernel instances that split the rows of one chunk (MS), with a
+# split that gets no row at all (M = 5 over 4 instances of 2 rows), and instances that walk heads (HB)
+TILED = [
+    ('cfg:rwkv7', '1,16,2,24,64', 'f32', 0, 'MS=4'),
+    ('cfg:mamba1', '2,16,2,5,16', 'f32', 1, 'MS=4'),
+    ('cfg:mamba2', '2,21,2,7,128', 'bf16', 1, 'MS=3'),
+    ('cfg:mamba2', '2,16,4,16,128', 'f32', 0, 'HB=2,MS=1'),
+    ('cfg:mamba2', '2,16,4,16,128', 'f32', 1, 'HB=4,MS=2'),
+]
+
+
+@pytest.mark.parametrize('case,dims,dtype,end,tile', TILED)
+def test_tile_overrides(case, dims, dtype, end, tile):
+    env = dict(os.environ, FLEX_RNN_TILE=tile)
+    r = subprocess.run([sys.executable, RUNNER, case, dims, dtype, str(end)], capture_output=True, text=True, timeout=900, env=env)
+    assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
+    assert tile.split(',')[0] in r.stdout.replace(' ', '')
+
+
 def _random_pattern_case(seed):
     """A gated linear-attention step whose five inputs get random classes-compatible broadcast
     patterns over (B, T, H); returns the argument string of run_case.py's `pattern:` mode."""
