@@ -9,6 +9,11 @@ noutputs, apply, forward_func, backward_func, fw_meta, bw_meta`, methods
 autograd formula, so the object composes with `torch.compile` without graph
 breaks.  Kernels are built lazily on the first real call; a later call with other
 shapes, strides or dtypes fails the metadata check, as in the reference.
+
+Beyond the reference: `jit(step, dynamic=True)` (or `jit.dynamic(step)`) keeps one plan per
+distinct (shape, stride, dtype) signature of the arguments instead of failing.  The kernels
+take B, T, H, M and all strides at run time, so signatures that lead to the same tile reuse
+the same cached code objects and only pay for tracing and planning.
 """
 from __future__ import annotations
 
@@ -24,10 +29,17 @@ def _tup(x):
     return x if type(x) == tuple else (x,)
 
 
+def _sig(tensors):
+    return tuple((tuple(int(n) for n in t.shape), tuple(int(n) for n in t.stride()), t.dtype) for t in tensors)
+
+
 class jit:
-    def __init__(self, step, n_step_args=None):
+    def __init__(self, step, n_step_args=None, dynamic=False):
         self.step = step
         self.forward_func = self.backward_func = None
+        self.is_dynamic = bool(dynamic)
+        self._entries = {}        # dynamic mode: argument signature -> plan entry
+        self._bw_index = {}       # dynamic mode: (input signature, checkpoint shapes) -> plan entry
         if n_step_args is None:
             n_step_args = len(inspect.signature(step).parameters)
         # arity: run the step once on 1x1 meta tensors (jit.py:13-16)
@@ -38,6 +50,32 @@ class jit:
 
     def __call__(self, *args):
         return self.apply(*args)
+
+    @classmethod
+    def dynamic(cls, step, n_step_args=None):
+        """Decorator form of `jit(step, dynamic=True)`."""
+        return cls(step, n_step_args, dynamic=True)
+
+    def _entry(self, inputs, state, dry):
+        """Dynamic mode: the plan entry for this argument signature, planned (`dry`) or built."""
+        key = _sig(inputs) + _sig(state)
+        e = self._entries.setdefault(key, {})
+        if dry:
+            if 'fw_meta' not in e:
+                e['fw_meta'], e['bw_meta'] = build_twopass(self.step, inputs, state, dryrun=True)
+        elif 'forward' not in e:
+            e['forward'], e['backward'], e['fw_meta'], e['bw_meta'] = build_twopass(self.step, inputs, state)
+        nout, nst = self.noutputs, self.nstates
+        stores = tuple(tuple(sh) for sh, _, _ in e['fw_meta'][nout + nst:nout + 2 * nst])
+        self._bw_index[_sig(inputs) + stores] = e
+        self.fw_meta, self.bw_meta = e['fw_meta'], e['bw_meta']
+        self.forward_func, self.backward_func = e.get('forward'), e.get('backward')
+        return e
+
+    def _bw_entry(self, inputs, state_store):
+        key = _sig(inputs) + tuple(tuple(int(n) for n in s.shape) for s in state_store)
+        assert key in self._bw_index, 'backward called with tensors no forward call has produced'
+        return self._bw_index[key]
 
     # ------------------------------------------------------------------ oracle
     def naive(self, *args, dtype=th.float32):
@@ -79,6 +117,11 @@ class jit:
         @th.library.custom_op('flex_rnn::fw_' + uid, mutates_args=(), schema=fw_schema)
         def apply(*args):
             inputs, state = split_list(args, [nin, nst])
+            if self.is_dynamic:
+                e = self._entry(inputs, state, dry=False)
+                r = e['forward'](inputs, state)
+                verify_meta(r, metas(e['fw_meta'], 'meta'))
+                return r
             if self.forward_func is None:
                 self.forward_func, self.backward_func, self.fw_meta, self.bw_meta = \
                     build_twopass(self.step, inputs, state)
@@ -89,6 +132,8 @@ class jit:
         @apply.register_fake
         def _(*args):
             inputs, state = split_list(args, [nin, nst])
+            if self.is_dynamic:
+                return metas(self._entry(inputs, state, dry=True)['fw_meta'], args[0].device)
             if not hasattr(self, 'fw_meta'):
                 self.fw_meta, self.bw_meta = build_twopass(self.step, inputs, state, dryrun=True)
             return metas(self.fw_meta, args[0].device)
@@ -99,12 +144,20 @@ class jit:
         @th.library.custom_op('flex_rnn::bw_' + uid, mutates_args=(), schema=bw_schema)
         def backward_inner(*args):
             doutput, dstateT, inputs, state_store, aux = split_list(args, [nout, nst, nin, nst, naux])
+            if self.is_dynamic:
+                e = self._bw_entry(inputs, state_store)
+                dinputs, dstate0 = e['backward'](doutput, dstateT, inputs, state_store, aux)
+                verify_meta(dinputs + dstate0, metas(e['bw_meta'], 'meta'))
+                return (*dinputs, *dstate0)
             dinputs, dstate0 = self.backward_func(doutput, dstateT, inputs, state_store, aux)
             verify_meta(dinputs + dstate0, metas(self.bw_meta, 'meta'))
             return (*dinputs, *dstate0)
 
         @backward_inner.register_fake
         def _(*args):
+            if self.is_dynamic:
+                _, _, inputs, state_store, _ = split_list(args, [nout, nst, nin, nst, naux])
+                return metas(self._bw_entry(inputs, state_store)['bw_meta'], args[0].device)
             return metas(self.bw_meta, args[0].device)
 
         def setup_context(ctx, inputs, output):

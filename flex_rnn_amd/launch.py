@@ -11,6 +11,7 @@ fp32 scratch + cast-back for gradients of inputs broadcast over batch / time / h
 from __future__ import annotations
 
 import struct
+from concurrent.futures import ThreadPoolExecutor
 from typing import Dict, List, Sequence, Tuple
 
 import torch as th
@@ -32,14 +33,18 @@ def kernel_specs(plan) -> List[KernelSpec]:
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
     """Emit + compile (or fetch from the cache) the three kernels.  Needs no GPU.  With
     `force` a cached code object is rebuilt, once per key recorded in `seen`."""
-    out = []
+    jobs = []
     for s in kernel_specs(plan):
         key = runtime.source_key(s.name, s.source)
         again = force and (seen is None or key not in seen)
         if seen is not None:
             seen.add(key)
-        out.append((s, runtime.compile_kernel(s.name, s.source, force=again)))
-    return out
+        jobs.append((s, again))
+    # the three compiler runs are independent processes: wait for them side by side (the
+    # runtime call releases the GIL)
+    with ThreadPoolExecutor(max_workers=len(jobs)) as pool:
+        paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
+    return [(s, path) for (s, _), path in zip(jobs, paths)]
 
 
 class CompiledPlan:

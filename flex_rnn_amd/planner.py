@@ -211,6 +211,23 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, HB=1, MS=MS)
 
 
+def check_tile(tile: TileConfig, H: int, N: int, part: Partition) -> None:
+    """Rejects a tile the kernels cannot run (an override is not trusted): the emitted index
+    arithmetic assumes every one of these."""
+    t = tile
+    for k in ('L', 'C', 'R', 'W', 'DT', 'TS', 'HB', 'MS'):
+        assert getattr(t, k) >= 1 and _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be a power of two'
+    for k in ('R1', 'W1'):
+        assert getattr(t, k) == 0 or _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be 0 or a power of two'
+    assert t.L <= 64 and t.L * t.C == N, f'tile covers {t.L}*{t.C} columns, the state has {N}'
+    assert t.W <= 16 and (t.W1 or t.W) <= 16, 'at most 16 waves per workgroup'
+    assert t.DT % t.TS == 0, 'the checkpoint interval must be a multiple of the staging depth'
+    assert not part.dstep_needs_state or t.TS == t.DT, \
+        'a reverse scan that recomputes the state stages a whole chunk (TS == DT)'
+    assert H % t.HB == 0, f'HB={t.HB} does not divide H={H}'
+    assert t.MS == 1 or part.epi_linear, 'rows can only be split (MS > 1) when the gradient epilogue is linear in the row sums'
+
+
 def part_input_classes(part: Partition) -> List[str]:
     cls = [None] * part.ninputs
     for name, idx in (('col', part.col_idx), ('row', part.row_idx), ('scalar', part.scalar_idx), ('mat', part.mat_idx)):
@@ -248,7 +265,7 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
         if override:
             import dataclasses
             tile = dataclasses.replace(tile, **{k: int(v) for k, v in (kv.split('=') for kv in override.split(','))})
-    assert tile.DT % tile.TS == 0
+    check_tile(tile, H, N, part)
     nchunks = -(-T // tile.DT)
     plan = Plan(B, T, H, M, N, part, cls, [i.dtype for i in inputs], bcast,
                 [s.dtype for s in state], [o.dtype for o in output_t], tile, nchunks)

@@ -94,6 +94,27 @@ def test_fake_tensor_mode_uses_dry_run():
     assert hasattr(f, 'fw_meta') and hasattr(f, 'bw_meta')
 
 
+def test_dynamic_mode_plans_one_entry_per_signature():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    f = flex_rnn_amd.jit.dynamic(ops.delta_rule)
+    assert f.is_dynamic and not flex_rnn_amd.jit(ops.delta_rule).is_dynamic
+    shapes = []
+    for dims in ((2, 16, 2, 8, 8), (1, 40, 2, 8, 8), (2, 16, 2, 8, 8)):
+        step, xs, ss = cases.make_inputs('delta_rule', *dims, dtype=th.float32)
+        with FakeTensorMode() as mode:
+            y, S = f(*[mode.from_tensor(x) for x in xs], *[mode.from_tensor(s) for s in ss])
+        shapes.append((tuple(y.shape), tuple(S.shape)))
+    assert shapes[0] == ((2, 16, 2, 8), (2, 2, 8, 8)) and shapes[1] == ((1, 40, 2, 8), (1, 2, 8, 8))
+    assert len(f._entries) == 2 and f.forward_func is None
+    # a strict instance keeps the first signature's metadata
+    g = flex_rnn_amd.jit(ops.delta_rule)
+    for dims in ((2, 16, 2, 8, 8), (1, 40, 2, 8, 8)):
+        step, xs, ss = cases.make_inputs('delta_rule', *dims, dtype=th.float32)
+        with FakeTensorMode() as mode:
+            y, S = g(*[mode.from_tensor(x) for x in xs], *[mode.from_tensor(s) for s in ss])
+    assert tuple(y.shape) == (2, 16, 2, 8)
+
+
 def test_compiled_path_has_no_cpu_fallback(runtime_lib):
     if th.cuda.is_available():
         pytest.skip('a GPU is present')

@@ -121,6 +121,26 @@ def test_second_call_with_other_shape_is_rejected():
         f(*_gpu(xs2), *_gpu(ss2))
 
 
+def test_dynamic_mode_accepts_other_shapes():
+    """`jit.dynamic`: batch, sequence length and strides change between calls; every call and its
+    gradients match the oracle, and calls of an earlier signature still work afterwards."""
+    print('case dynamic signatures', flush=True)
+    f = flex_rnn_amd.jit.dynamic(ops.gla)
+    for dims in ((1, 16, 2, 16, 16), (3, 50, 2, 16, 16), (1, 16, 2, 16, 16), (2, 33, 2, 16, 16)):
+        step, xs, ss = cases.make_inputs('gla', *dims, dtype=th.float32)
+        gx = [x.requires_grad_() for x in _gpu(xs)]
+        gs = [s_.requires_grad_() for s_ in _gpu(ss)]
+        out = f(*gx, *gs)
+        g = th.Generator().manual_seed(5)
+        dys = [th.randn(o.shape, generator=g) for o in out]
+        grads = th.autograd.grad(out, gx + gs, [d.cuda() for d in dys])
+        want = recurrence.loop_with_grads(step, xs, ss, dys[:1], dys[1:], dtype=th.float64)
+        ref = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+        for a, b in zip(list(out) + list(grads), ref):
+            assert recurrence.rel_err(a, b) < 1e-4, dims
+    assert len(f._entries) == 3
+
+
 def test_torch_compile_no_graph_break():
     print('case torch.compile', flush=True)
     step, xs, ss = cases.make_inputs('delta_rule', 2, 32, 2, 16, 16, dtype=th.float32)
