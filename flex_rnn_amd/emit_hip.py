@@ -89,6 +89,7 @@ template <> __device__ __forceinline__ void stf<3>(void* p, i64 i, float v) { ((
 __device__ __forceinline__ void atomic_addf(void* p, i64 i, float v) {
   __hip_atomic_fetch_add(((float*)p) + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ float f_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float f_sigmoid(float x) { return 1.0f / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float f_tanh(float x) { return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f); }
 __device__ __forceinline__ float f_sign(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f); }
@@ -141,11 +142,18 @@ def _loops(rr, cc):
 
 
 def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple[bool, bool]],
-                  reduce_fn: str) -> Tuple[str, List[str]]:
+                  reduce_fn: str, invariant: Sequence[str] = ()) -> Tuple[str, List[str]]:
     """Device function evaluating `g` on register tiles.  Every value is a `float[RR][CC]`
     array with RR = R if it varies along rows else 1, CC likewise for columns.  Returns the
-    source and the list of graph inputs that appear in the signature (the used ones)."""
+    source and the list of graph inputs that appear in the signature (the used ones).
+
+    `invariant` names graph inputs that do not change from one timestep to the next.
+    `exp(u * v)` with such a `v` is evaluated as `exp2(u * (v * log2 e))`: the hardware
+    exponential is base 2, and the rescaled `v` is loop-invariant for the compiler to hoist,
+    which saves the multiply by log2 e on every step."""
     ext = g.ext_table()
+    nm = g.node_map()
+    invariant = set(invariant)
     used = [i for i, u in zip(g.inputs, g.used_inputs()) if u]
     params = [_ref(i, g.input_ext[i], R, C, True) for i in used]
     params += [_ref(f'o{k}_', e, R, C, False) for k, e in enumerate(out_exts)]
@@ -170,6 +178,12 @@ def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple
                        f'    {n.name}[r][0] = {reduce_fn}(s_);\n  }}')
         elif n.op == 'const':
             out.append(f'  {n.name}[0][0] = {_lit(n.args[0])};')
+        elif n.op == 'exp' and isinstance(n.args[0], str) and n.args[0] in nm and nm[n.args[0]].op == 'mul' \
+                and any(a in invariant for a in nm[n.args[0]].value_args()) and len(nm[n.args[0]].value_args()) == 2:
+            u, v = nm[n.args[0]].args
+            if u in invariant:
+                u, v = v, u
+            out.append('  ' + _loops(rr, cc) + f'{n.name}[r][c] = f_exp2({opnd(u)} * ({opnd(v)} * 1.4426950408889634f));')
         elif n.op in _UNARY_EXPR:
             out.append('  ' + _loops(rr, cc) + f'{n.name}[r][c] = ' + _UNARY_EXPR[n.op].format(opnd(n.args[0])) + ';')
         elif n.op in _BINARY_EXPR:
@@ -309,6 +323,7 @@ class Emitter:
         # (when T == 1 every non-matrix input counts as time-dependent, with a single step)
         self.tdep = [(plan.T == 1 or not b[1]) and c != 'mat' for b, c in zip(plan.in_bcast, self.cls)]
         self.atomic = set(plan.atomic)
+        self.invariant = {nm for nm, td in zip(p.in_names, self.tdep) if not td}
         self.jext = p.joint.ext_table()
         # the last chunk is partial when T is not a multiple of the chunk sizes; the guards that
         # handles it are only emitted then, so aligned lengths keep the unguarded code
@@ -399,7 +414,7 @@ class Emitter:
         # a state of a problem with M == 1 or N == 1 has a smaller extent; follow the joint graph
         st_ext = [self.jext[s] for s in p.st_names]
         out_exts = [(st_ext[0][0], False)] * nout + st_ext + [(st_ext[0][0], False)] * naux
-        fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>')
+        fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
         used_in = [i for i in range(nin) if p.in_names[i] in used]
         src, MT = self._row_kernel_common(R, W)
         body = []
@@ -513,12 +528,12 @@ class Emitter:
         g = p.dstep
         mats = list(p.mat_idx) if p.mat_in_dstep else []
         out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux + [(True, True)] * len(mats)
-        fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>')
+        fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
         fns = [fn_src]
         used_all = set(used)
         re_used = []
         if needs_state:
-            re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>')
+            re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>', self.invariant)
             fns.append(re_src)
             used_all |= set(re_used)
         used_in = [i for i in range(nin) if p.in_names[i] in used_all]
@@ -577,12 +592,21 @@ class Emitter:
         body.append('    __syncthreads();\n')
         body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ') + '    }\n')
 
+        # With state recompute a timestep's operands are read by `bw_restep` and again by
+        # `bw_dstep`.  Those without a column extent (one register per row) are loaded once for
+        # both, so that the compiler sees common subexpressions of the two calls - typically
+        # the exponential of a per-row decay - as such.
+        shared_in = [i for i in used_in if needs_state and self.tdep[i] and not self.in_ext(i)[1]
+                     and p.in_names[i] in used and p.in_names[i] in re_used]
+
         def operand_loads(tt, names, state_var):
             code, call = [], []
             for nm_ in names:
                 if nm_ in p.in_names:
                     i = p.in_names.index(nm_)
-                    if self.tdep[i]:
+                    if i in shared_in:
+                        call.append(f'x{i}_{tt}')
+                    elif self.tdep[i]:
                         code.append(self._load_operand(f'x{i}_{tt}' if needs_state else f'x{i}', f's_in{i}', self.in_ext(i), R, C, tt))
                         call.append(f'x{i}_{tt}' if needs_state else f'x{i}')
                     else:
@@ -653,6 +677,9 @@ class Emitter:
                 for k in range(nst):
                     rr, cc = _dims(st_ext[k], R, C)
                     body.append(f'    float Sh{k}_{tt}[{rr}][{cc}];\n')
+            for tt in range(DT):
+                for i in shared_in:
+                    body.append(self._load_operand(f'x{i}_{tt}', f's_in{i}', self.in_ext(i), R, C, str(tt)))
             for tt in range(DT - 1):
                 body.append(f'    if ({tt + 1} < nt) {{\n' if tail else '    {\n')
                 code, call = operand_loads(str(tt), re_used, lambda k, tt=tt: f'Sh{k}_{tt}')
@@ -726,8 +753,8 @@ class Emitter:
         op_names = [nm_[m].args[0] for m in p.msums]
         mats2 = [] if p.mat_in_dstep else list(p.mat_idx)
         drow_exts = st_ext + [(True, True)] * len(mats2) + [self.jext[o] for o in op_names]
-        drow_src, drow_used = emit_graph_fn(p.drow, 'bw_drow', 1, 1, drow_exts, red)
-        re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', 1, 1, st_ext, red)
+        drow_src, drow_used = emit_graph_fn(p.drow, 'bw_drow', 1, 1, drow_exts, red, self.invariant)
+        re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', 1, 1, st_ext, red, self.invariant)
         epi_exts = [self.in_ext(i) for i in rs]
         epi_src, epi_used = emit_graph_fn(p.epi, 'bw_epi', 1, 1, epi_exts, red)
         loop_used = set(drow_used) | set(re_used)

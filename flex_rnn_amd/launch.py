@@ -25,9 +25,17 @@ def _strides5(t: th.Tensor) -> Tuple[int, ...]:
     return tuple(s + [0] * (5 - len(s)))
 
 
+def needs_gradient_kernel(plan) -> bool:
+    """The per-chunk gradient kernel produces the row- and scalar-input gradients and, unless the
+    reverse scan already does, the matrix-input gradients.  A recurrence with none of these
+    (all inputs per-row, e.g. a vector state) is finished after the reverse scan."""
+    p = plan.part
+    return bool(p.row_idx or p.scalar_idx or (p.mat_idx and not p.mat_in_dstep))
+
+
 def kernel_specs(plan) -> List[KernelSpec]:
     em = Emitter(plan)
-    return [em.fw(), em.bw1(), em.bw2()]
+    return [em.fw(), em.bw1()] + ([em.bw2()] if needs_gradient_kernel(plan) else [])
 
 
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
@@ -150,7 +158,8 @@ class CompiledPlan:
         for k in range(p.noutputs):
             tensors[f'dout{k}'] = doutput[k]
         self._launch('frnn_bw1', tensors)
-        self._launch('frnn_bw2', tensors)
+        if 'frnn_bw2' in self.kernels:
+            self._launch('frnn_bw2', tensors)
         for i in atomic:
             x = inputs[i]
             g = th.empty_like(x)

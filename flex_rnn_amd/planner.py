@@ -215,8 +215,9 @@ def check_tile(tile: TileConfig, H: int, N: int, part: Partition) -> None:
     """Rejects a tile the kernels cannot run (an override is not trusted): the emitted index
     arithmetic assumes every one of these."""
     t = tile
-    for k in ('L', 'C', 'R', 'W', 'DT', 'TS', 'HB', 'MS'):
+    for k in ('L', 'C', 'R', 'W', 'DT', 'TS'):
         assert getattr(t, k) >= 1 and _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be a power of two'
+    assert t.HB >= 1 and 1 <= t.MS <= 65535, 'HB and MS must be positive (MS is a grid dimension)'
     for k in ('R1', 'W1'):
         assert getattr(t, k) == 0 or _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be 0 or a power of two'
     assert t.L <= 64 and t.L * t.C == N, f'tile covers {t.L}*{t.C} columns, the state has {N}'
