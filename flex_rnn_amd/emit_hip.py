@@ -733,7 +733,9 @@ class Emitter:
         return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
 
     # ------------------------------------------------------------------ bw2
-    def bw2(self) -> KernelSpec:
+    def bw2(self, waves_per_simd: int = 0) -> KernelSpec:
+        """`waves_per_simd` > 0 asks the compiler to fit that many waves on a SIMD (fewer registers,
+        possibly spills); the caller compares the outcomes."""
         p, plan, t = self.p, self.plan, self.tile
         N, DT = plan.N, t.DT
         IPB = max(1, 64 // N)
@@ -752,13 +754,36 @@ class Emitter:
         red = f'inst_allreduce<{N}>'
         op_names = [nm_[m].args[0] for m in p.msums]
         mats2 = [] if p.mat_in_dstep else list(p.mat_idx)
-        drow_exts = st_ext + [(True, True)] * len(mats2) + [self.jext[o] for o in op_names]
-        drow_src, drow_used = emit_graph_fn(p.drow, 'bw_drow', 1, 1, drow_exts, red, self.invariant)
-        re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', 1, 1, st_ext, red, self.invariant)
+        # Per-row scalars.  A value with a row extent but no column extent is the same on every
+        # lane of an instance; the row loop would recompute it on each of them for every
+        # (row, timestep).  The outermost such values (`front`: those feeding a full-tile value or
+        # a row sum) are instead evaluated where the chunk's per-row operands are staged, one
+        # (row, timestep) per lane, and reach the row loop through LDS like a raw operand.  A row
+        # sum of such a value (`colsum`) never enters the row loop: it is summed from LDS.
+        front = []
+        # (a vector state, N == 1, has no column extent itself: nothing to tell apart there)
+        for g_ in ((p.restep, p.drow) if all(e[1] for e in st_ext) else ()):
+            for n_ in g_.nodes:
+                if n_.ext == (True, False) and n_.name not in front and (
+                        n_.name in g_.outputs or any(n_.name in m_.value_args() and m_.ext[1] for m_ in g_.nodes)):
+                    front.append(n_.name)
+        colsum = [j for j, o in enumerate(op_names) if o in front]
+        loop_ops = [j for j in range(len(op_names)) if j not in colsum]
+        restep_g = p.restep.extract('restep', p.restep.outputs, cut=front) if front else p.restep
+        drow_outs = list(p.drow.outputs[:nst + len(mats2)]) + [op_names[j] for j in loop_ops]
+        drow_g = p.drow.extract('drow', drow_outs, cut=front) if front else p.drow
+        drow_exts = st_ext + [(True, True)] * len(mats2) + [self.jext[op_names[j]] for j in loop_ops]
+        drow_src, drow_used = emit_graph_fn(drow_g, 'bw_drow', 1, 1, drow_exts, red, self.invariant)
+        re_src, re_used = emit_graph_fn(restep_g, 'bw_restep', 1, 1, st_ext, red, self.invariant)
         epi_exts = [self.in_ext(i) for i in rs]
         epi_src, epi_used = emit_graph_fn(p.epi, 'bw_epi', 1, 1, epi_exts, red)
         loop_used = set(drow_used) | set(re_used)
         all_used = loop_used | set(epi_used)
+        pre_src, pre_used = '', []
+        if front:
+            cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
+            pre_g = p.joint.extract('colpre', front, cut=set(cuts))
+            pre_src, pre_used = emit_graph_fn(pre_g, 'bw_colpre', 1, 1, [(True, False)] * len(front), red, self.invariant)
 
         def is_rowlike(nm):      # no row extent: can be loaded once per chunk
             return not self.jext[nm][0]
@@ -829,6 +854,28 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         def aux_load(k, tt, mexpr):
             return f'((const float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + ({tclamp(tt)})) * M + {mexpr}]'
 
+        def raw_value(v, tt, mexpr):
+            """Global-memory value of graph input `v` (an input, saved sum or output gradient without
+            a column extent) at timestep offset `tt` of the chunk and row `mexpr`."""
+            if v in p.in_names:
+                i = p.in_names.index(v)
+                ext = self.in_ext(i)
+                assert not ext[1], v
+                dt = DT_CODE[plan.in_dtypes[i]]
+                idx = self._in_index(A, i, t=(tclamp(tt) if self.tdep[i] else '0'), m=(mexpr if ext[0] else None))
+                return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
+            if v in p.aux:
+                return aux_load(p.aux.index(v), tt, mexpr if self.jext[v][0] else '0')
+            if v in p.daux:
+                return f'((const float*){A.p("daux")})[((((i64){p.daux.index(v)} * A.B + b) * H + h) * T + ({tclamp(tt)})) * M + {mexpr}]'
+            if v in p.dout_names:
+                k = p.dout_names.index(v)
+                dt = DT_CODE[plan.out_dtypes[k]]
+                nmv = f'dout{k}'
+                return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)({tclamp(tt)}) * {A.s(nmv, 1)} + '
+                        f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
+            raise AssertionError(v)
+
         # ---- per-chunk loads of everything without a row extent
         for i in range(nin):
             if p.in_names[i] not in all_used or self.in_ext(i)[0]:
@@ -842,7 +889,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             if p.aux[k] in all_used and is_rowlike(p.aux[k]):
                 for tt in range(DT):
                     b.append(f'  float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "0")};\n')
-        for j in range(len(p.msums)):
+        for j in loop_ops:
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
         # ---- per-row operands of the chunk go through LDS: staged once per row block by the
@@ -871,6 +918,15 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     return (f'ldf<{dt}>({A.p(nmv)}, (i64)b * {A.s(nmv, 0)} + (i64)({tclamp(tt)}) * {A.s(nmv, 1)} + '
                             f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
                 rowops.append((f's_dy{k}', ldy, f'dy{k}'))
+        for q in range(len(front)):
+            rowops.append((f's_f{q}', None, f'f{q}'))
+        for j in colsum:
+            b.append(f'  __shared__ float s_cs{j}[{IPB}][{DT}];\n')
+        if colsum:
+            if HB > 1:
+                b.append('  __syncthreads();\n')
+            b.append(f'  for (int tt_ = n; tt_ < {DT}; tt_ += {min(N, NT)}) {{ '
+                     + ' '.join(f's_cs{j}[inst][tt_] = 0.0f;' for j in colsum) + ' }\n')
         MB = 1
         while MB * 2 <= MR and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
             MB *= 2
@@ -894,8 +950,27 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append(f'#pragma unroll {min(trips, 2)}\n    for (int i_ = 0; i_ < {trips}; i_++) {{ const int e_ = n + i_ * {lanes}; {guard}{{ '
                      f'const int tt_ = e_ / {MB}, mm_ = e_ % {MB}; const int mc_ = min(m0 + mm_, M - 1);\n')
             for nm_lds, ld, _ in rowops:
-                b.append(f'      {nm_lds}[inst][mm_][tt_] = {ld("tt_", "mc_")};\n')
+                if ld is not None:
+                    b.append(f'      {nm_lds}[inst][mm_][tt_] = {ld("tt_", "mc_")};\n')
+            if front:
+                call = []
+                for v in pre_used:
+                    b.append(f'      float p_{v}[1][1]; p_{v}[0][0] = {raw_value(v, "tt_", "mc_")};\n')
+                    call.append(f'p_{v}')
+                for q in range(len(front)):
+                    b.append(f'      float pf{q}[1][1];\n')
+                    call.append(f'pf{q}')
+                b.append('      bw_colpre(' + ', '.join(call) + ');\n')
+                for q in range(len(front)):
+                    b.append(f'      s_f{q}[inst][mm_][tt_] = pf{q}[0][0];\n')
             b.append('    } }\n    __syncthreads();\n')
+            if colsum:
+                cond = f'if (tt_ < nt) ' if tail else ''
+                b.append(f'    for (int tt_ = n; tt_ < {DT}; tt_ += {lanes}) {cond}{{ const int nv_ = min({MB}, mhi - m0);\n')
+                for j in colsum:
+                    q = front.index(op_names[j])
+                    b.append(f'      {{ float a_ = 0.0f; for (int mm_ = 0; mm_ < nv_; mm_++) a_ += s_f{q}[inst][mm_][tt_]; s_cs{j}[inst][tt_] += a_; }}\n')
+                b.append('    }\n')
         b.append(f'#pragma unroll {min(PD, MB)}\n  for (int mm = 0; mm < {MB}; mm++) {{\n    const int m = m0 + mm;\n    if (m >= mhi) break;\n')
         for k in range(nst):
             b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Sq{k}_0;\n')
@@ -909,7 +984,9 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append(f'      Sq{k}_{PD - 1} = sckp{k}[mn_ * {N}];\n')
             b.append(f'      Dq{k}_{PD - 1} = dckp{k}[mn_ * {N}];\n')
         b.append('    }\n')
-        for nm_lds, _, pref in rowops:
+        for nm_lds, ld, pref in rowops:
+            if ld is None and front[int(pref[1:])] not in loop_used:
+                continue                    # only summed over rows, never read by the row loop
             for tt in range(DT):
                 b.append(f'    float {pref}_{tt}[1][1]; {pref}_{tt}[0][0] = {nm_lds}[inst][mm][{tt}];\n')
         for i in range(nin):
@@ -935,6 +1012,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     call.append(f'D{p.dnst_names.index(v)}')
                 elif v in p.msums:
                     call.append(f'ms{p.msums.index(v)}')
+                elif v in front:
+                    call.append(f'f{front.index(v)}_{tt}')
                 else:
                     raise AssertionError(v)
             return call
@@ -955,7 +1034,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             for i in mats2:
                 b.append(f'      float gm{i}[1][1];\n')
                 call.append(f'gm{i}')
-            for j in range(len(p.msums)):
+            for j in loop_ops:
                 b.append(f'      float op{j}[1][1];\n')
                 call.append(f'op{j}')
             b.append('      bw_drow(' + ', '.join(call) + ');\n')
@@ -963,7 +1042,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                 b.append(f'      D{k}[0][0] = nD{k}[0][0];\n')
             for i in mats2:
                 b.append(f'      ma{i} += gm{i}[0][0];\n')
-            for j in range(len(p.msums)):
+            for j in loop_ops:
                 b.append(f'      acc{j}_{tt} += op{j}[0][0];\n')
             b.append('    }\n')
         for i in mats2:
@@ -999,6 +1078,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         nred = [j for j, mname in enumerate(p.msums)
                 if 1 in nm_[mname].dims and self.jext[nm_[mname].args[0]][1]]
         batched = N > 64 and bool(nred)
+        if colsum:
+            b.append('  __syncthreads();\n')
         if batched:
             NW = N // 64
             b.append(f'  __shared__ float red_ms[{len(nred) * DT}][{NW}];\n')
@@ -1020,6 +1101,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                 opext = self.jext[node.args[0]]
                 if 1 in node.dims and opext[1] and not batched:
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}(acc{j}_{tt});\n')
+                elif j in colsum:
+                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = s_cs{j}[inst][{tt}];\n')
                 else:
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = acc{j}_{tt};\n')
             call = call_args(epi_used, tt, None)
@@ -1047,6 +1130,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             else:
                 for tt in range(DT):
                     b.append(write_out(i, tt, 'h0', f'gh{i}_{tt}', '  '))
-        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
-        source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + kernel
+        wpe = int(waves_per_simd)
+        attr = f' __attribute__((amdgpu_waves_per_eu({wpe},{wpe})))' if wpe else ''
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){attr} frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
+        source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + pre_src + '\n' + kernel
         return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})', str(MS)))

@@ -38,21 +38,41 @@ def kernel_specs(plan) -> List[KernelSpec]:
     return [em.fw(), em.bw1()] + ([em.bw2()] if needs_gradient_kernel(plan) else [])
 
 
+MAX_SPILL_BYTES = 64      # per lane; beyond this a higher-occupancy build of the gradient kernel is not taken
+
+
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
-    """Emit + compile (or fetch from the cache) the three kernels.  Needs no GPU.  With
-    `force` a cached code object is rebuilt, once per key recorded in `seen`."""
-    jobs = []
-    for s in kernel_specs(plan):
-        key = runtime.source_key(s.name, s.source)
-        again = force and (seen is None or key not in seen)
-        if seen is not None:
-            seen.add(key)
-        jobs.append((s, again))
-    # the three compiler runs are independent processes: wait for them side by side (the
-    # runtime call releases the GIL)
-    with ThreadPoolExecutor(max_workers=len(jobs)) as pool:
-        paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
-    return [(s, path) for (s, _), path in zip(jobs, paths)]
+    """Emit + compile (or fetch from the cache) the kernels of a plan.  Needs no GPU.  With
+    `force` a cached code object is rebuilt, once per key recorded in `seen`.
+
+    The gradient kernel is register-hungry (a chunk of accumulators per lane) and hides memory
+    latency only through the waves resident on its SIMD.  After the plain build, builds that ask
+    the compiler for one more wave per SIMD are tried, and taken as long as they spill at most
+    `MAX_SPILL_BYTES` per lane; the compiler's own resource report decides, not a timing."""
+    def build(specs):
+        jobs = []
+        for s in specs:
+            key = runtime.source_key(s.name, s.source)
+            again = force and (seen is None or key not in seen)
+            if seen is not None:
+                seen.add(key)
+            jobs.append((s, again))
+        # independent compiler processes: wait for them side by side (the runtime call releases the GIL)
+        with ThreadPoolExecutor(max_workers=max(1, len(jobs))) as pool:
+            paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
+        return [(s, path) for (s, _), path in zip(jobs, paths)]
+
+    built = build(kernel_specs(plan))
+    if built[-1][0].name == 'frnn_bw2':
+        res = runtime.kernel_resources(built[-1][1])
+        em = Emitter(plan)
+        while res is not None and res['occupancy'] < 4 and res['vgprs'] <= 224:
+            cand = build([em.bw2(waves_per_simd=res['occupancy'] + 1)])[0]
+            cres = runtime.kernel_resources(cand[1])
+            if cres is None or cres['occupancy'] <= res['occupancy'] or cres['scratch'] > MAX_SPILL_BYTES:
+                break
+            built[-1], res = cand, cres
+    return built
 
 
 class CompiledPlan:

@@ -8,7 +8,9 @@ from __future__ import annotations
 
 import ctypes
 import hashlib
+import json
 import os
+import re
 import subprocess
 from typing import Sequence
 
@@ -16,7 +18,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)
 LIB_PATH = os.path.join(_HERE, 'libfrnn_rt.so')
 ARCH = 'gfx950'
-EMITTER_OPTS = '-ffp-contract=fast -munsafe-fp-atomics'
+# (the resource-usage remarks land in the compile log; `kernel_resources` reads them back)
+EMITTER_OPTS = '-ffp-contract=fast -munsafe-fp-atomics -Rpass-analysis=kernel-resource-usage'
 
 _lib = None
 
@@ -116,7 +119,47 @@ def compile_kernel(name: str, src: str, opts: str = EMITTER_OPTS, force: bool = 
     b = src.encode()
     rc = lib().frnn_compile(b, len(b), ARCH.encode(), opts.encode(), cache_dir().encode(), key.encode(), out, 4096)
     _check(rc, f'compiling kernel {name}')
-    return out.value.decode()
+    path = out.value.decode()
+    _record_resources(path)
+    return path
+
+
+_RES_FIELDS = {'vgprs': r'\bVGPRs: (\d+)', 'scratch': r'ScratchSize \[bytes/lane\]: (\d+)',
+               'occupancy': r'Occupancy \[waves/SIMD\]: (\d+)', 'lds': r'LDS Size \[bytes/block\]: (\d+)'}
+
+
+def _record_resources(hsaco: str) -> None:
+    """After a compile, condenses the compiler's resource-usage remarks (registers, spill bytes,
+    waves per SIMD, LDS) into `<key>.res` next to the code object; the log itself need not be
+    kept."""
+    base = hsaco[:-len('.hsaco')]
+    if os.path.exists(base + '.res') and os.path.getmtime(base + '.res') >= os.path.getmtime(hsaco):
+        return
+    try:
+        with open(base + '.log') as f:
+            log = f.read()
+    except OSError:
+        return
+    vals = {}
+    for k, pat in _RES_FIELDS.items():
+        m = re.search(pat, log)
+        if m:
+            vals[k] = int(m.group(1))
+    if len(vals) == len(_RES_FIELDS):
+        tmp = f'{base}.res.tmp{os.getpid()}'
+        with open(tmp, 'w') as f:
+            json.dump(vals, f)
+        os.replace(tmp, base + '.res')
+
+
+def kernel_resources(hsaco: str):
+    """{'vgprs', 'scratch' (spill bytes per lane), 'occupancy' (waves per SIMD), 'lds'} of a
+    compiled kernel, or None when unknown."""
+    try:
+        with open(hsaco[:-len('.hsaco')] + '.res') as f:
+            return json.load(f)
+    except (OSError, ValueError):
+        return None
 
 
 class Kernel:
