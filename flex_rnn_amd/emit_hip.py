@@ -248,9 +248,19 @@ class _Stager:
     def __init__(self, TS: int, NT: int, tail: bool = False):
         self.TS, self.NT, self.tail = TS, NT, tail
         self.items = []      # (lds name, row length, dtype code, pointer, index fn(t, x_), time stride)
+        self.no_lds = set()  # items that only feed derived operands: prefetched, never written to LDS
+        self.derived = None  # (function name, [source item names], [derived lds names], row length)
 
-    def add(self, name, ln, dt, ptr, idx_fn, tstride):
+    def add(self, name, ln, dt, ptr, idx_fn, tstride, lds=True):
         self.items.append((name, ln, dt, ptr, idx_fn, tstride))
+        if not lds:
+            self.no_lds.add(name)
+
+    def derive(self, fn_name, sources, outputs, ln):
+        """Operands computed while staging: `fn_name(src..., out...)` is evaluated once per
+        (timestep, position) from the converted prefetch registers of `sources` (items of row
+        length `ln`) and its results are written to the LDS arrays `outputs`."""
+        self.derived = (fn_name, list(sources), list(outputs), ln)
 
     def _iters(self, ln):
         return (self.TS * ln + self.NT - 1) // self.NT
@@ -261,7 +271,12 @@ class _Stager:
     def decls(self) -> str:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
-            out += f'  __shared__ float {name}[{self.TS}][{ln}];\n  unsigned pf_{name}[{self._iters(ln)}];\n'
+            if name not in self.no_lds:
+                out += f'  __shared__ float {name}[{self.TS}][{ln}];\n'
+            out += f'  unsigned pf_{name}[{self._iters(ln)}];\n'
+        if self.derived:
+            for o in self.derived[2]:
+                out += f'  __shared__ float {o}[{self.TS}][{self.derived[3]}];\n'
         return out
 
     def bases(self) -> str:
@@ -299,7 +314,16 @@ class _Stager:
     def write(self, ind: str) -> str:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
-            out += self._loop(ln, f'{name}[tt_][x_] = cvr<{dt}>(pf_{name}[it_]);', ind)
+            if name not in self.no_lds:
+                out += self._loop(ln, f'{name}[tt_][x_] = cvr<{dt}>(pf_{name}[it_]);', ind)
+        if self.derived:
+            fn_name, sources, outputs, ln = self.derived
+            dts = {name: dt for name, _, dt, _, _, _ in self.items}
+            body = '{ ' + ' '.join(f'float a{k}_[1][1]; a{k}_[0][0] = cvr<{dts[s_]}>(pf_{s_}[it_]);' for k, s_ in enumerate(sources))
+            body += ' ' + ' '.join(f'float d{k}_[1][1];' for k in range(len(outputs)))
+            body += f' {fn_name}(' + ', '.join([f'a{k}_' for k in range(len(sources))] + [f'd{k}_' for k in range(len(outputs))]) + ');'
+            body += ' ' + ' '.join(f'{o}[tt_][x_] = d{k}_[0][0];' for k, o in enumerate(outputs)) + ' }'
+            out += self._loop(ln, body, ind)
         return out
 
 
@@ -344,6 +368,49 @@ class Emitter:
         return ' + '.join(terms)
 
     # ------------------------------------------------------------------ row kernels
+    def _row_front(self, graphs):
+        """Row operands that can be computed while staging.  In the row kernels a value with a
+        column but no row extent (a function of a timestep's row inputs: the exponential of a
+        log-decay, a gate's sigmoid, a normalised key) would be recomputed by every row group of
+        every wave.  Returns the outermost such values that depend on nothing but staged row
+        inputs and constants; the staging threads evaluate them once per (timestep, column)."""
+        p = self.p
+        ok = {p.in_names[i] for i in range(p.ninputs) if self.tdep[i] and self.in_ext(i) == (False, True)}
+        front = []
+        for g in graphs:
+            consts, pure = set(), set()
+            for n in g.nodes:
+                args = n.value_args()
+                if n.op == 'const' or (n.op != 'sum' and n.ext == (False, False) and args and all(a in consts for a in args)):
+                    consts.add(n.name)
+                elif n.op != 'sum' and n.ext == (False, True) and all(a in ok or a in pure or a in consts for a in args) \
+                        and any(a in ok or a in pure for a in args):
+                    pure.add(n.name)
+            for n in g.nodes:
+                if n.name in pure and n.name not in front and (
+                        n.name in g.outputs or any(n.name in m.value_args() and m.name not in pure for m in g.nodes)):
+                    front.append(n.name)
+        return front
+
+    def _stage_row_front(self, stg: '_Stager', A: _Args, front, direct_used, MT: int, fn_name: str):
+        """Registers the raw inputs the derived operands need (without an LDS array of their own
+        unless the step function also reads them directly) and the derivation itself; returns the
+        source of the device function."""
+        p = self.p
+        pre_g = p.joint.extract(fn_name, front, cut=())
+        src, used = emit_graph_fn(pre_g, fn_name, 1, 1, [(False, True)] * len(front), 'grp_allreduce<1>')
+        have = {it[0] for it in stg.items}
+        for v in used:
+            i = p.in_names.index(v)
+            if f's_in{i}' not in have:
+                ext = self.in_ext(i)
+                assert ext == (False, True)
+                dt = DT_CODE[self.plan.in_dtypes[i]]
+                stg.add(f's_in{i}', self.plan.N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x),
+                        A.s(f'in{i}', 1), lds=p.in_names[i] in direct_used)
+        stg.derive(fn_name, [f's_in{p.in_names.index(v)}' for v in used], [f's_d{q}' for q in range(len(front))], self.plan.N)
+        return src
+
     def _row_kernel_common(self, R: int, W: int):
         """Declarations shared by fw and bw1: thread mapping and staging buffers."""
         t = self.tile
@@ -414,6 +481,9 @@ class Emitter:
         # a state of a problem with M == 1 or N == 1 has a smaller extent; follow the joint graph
         st_ext = [self.jext[s] for s in p.st_names]
         out_exts = [(st_ext[0][0], False)] * nout + st_ext + [(st_ext[0][0], False)] * naux
+        rfront = self._row_front([g])
+        if rfront:
+            g = g.extract('fw', g.outputs, cut=rfront)
         fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
         used_in = [i for i in range(nin) if p.in_names[i] in used]
         src, MT = self._row_kernel_common(R, W)
@@ -424,6 +494,8 @@ class Emitter:
         for i in used_in:
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
+        if rfront:
+            fn_src = self._stage_row_front(stg, A, rfront, set(used), MT, 'fw_rowpre') + '\n' + fn_src
         body.append(stg.decls() + stg.bases())
         for k in range(nout):
             body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
@@ -464,6 +536,10 @@ class Emitter:
                 call.append(f'x{i}')
             elif nm_ in p.st_names:
                 call.append(f'S{p.st_names.index(nm_)}')
+            elif nm_ in rfront:
+                q = rfront.index(nm_)
+                body.append(self._load_operand(f'd{q}', f's_d{q}', (False, True), R, C, 'tt'))
+                call.append(f'd{q}')
             else:
                 raise AssertionError(nm_)
         rrs = R if st_ext[0][0] else 1
@@ -528,12 +604,17 @@ class Emitter:
         g = p.dstep
         mats = list(p.mat_idx) if p.mat_in_dstep else []
         out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux + [(True, True)] * len(mats)
+        restep_g = p.restep
+        rfront = self._row_front([g, restep_g] if needs_state else [g])
+        if rfront:
+            g = g.extract('dstep', g.outputs, cut=rfront)
+            restep_g = restep_g.extract('restep', restep_g.outputs, cut=rfront)
         fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
         fns = [fn_src]
         used_all = set(used)
         re_used = []
         if needs_state:
-            re_src, re_used = emit_graph_fn(p.restep, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>', self.invariant)
+            re_src, re_used = emit_graph_fn(restep_g, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>', self.invariant)
             fns.append(re_src)
             used_all |= set(re_used)
         used_in = [i for i in range(nin) if p.in_names[i] in used_all]
@@ -554,6 +635,8 @@ class Emitter:
             stg.add(f's_dy{k}', MT, DT_CODE[plan.out_dtypes[k]], A.p(nm),
                     lambda tt, x, nm=nm: (f'(i64)b * {A.s(nm, 0)} + (i64)({tt}) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + '
                                            f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'), A.s(nm, 1))
+        if rfront:
+            fns.insert(0, self._stage_row_front(stg, A, rfront, used_all, MT, 'bw_rowpre'))
         body.append(stg.decls() + stg.bases())
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
@@ -626,6 +709,11 @@ class Emitter:
                     call.append(v)
                 elif nm_ in p.dnst_names:
                     call.append(f'D{p.dnst_names.index(nm_)}')
+                elif nm_ in rfront:
+                    q = rfront.index(nm_)
+                    v = f'd{q}_{tt}' if needs_state else f'd{q}'
+                    code.append(self._load_operand(v, f's_d{q}', (False, True), R, C, tt))
+                    call.append(v)
                 else:
                     raise AssertionError(nm_)
             return code, call
@@ -769,21 +857,39 @@ class Emitter:
                     front.append(n_.name)
         colsum = [j for j, o in enumerate(op_names) if o in front]
         loop_ops = [j for j in range(len(op_names)) if j not in colsum]
-        restep_g = p.restep.extract('restep', p.restep.outputs, cut=front) if front else p.restep
+        # Row-invariant values (no row extent: functions of the row / scalar inputs of a timestep,
+        # e.g. the exponential of a log-decay) are the same for every row of the chunk.  The
+        # outermost ones (`rfront`) are evaluated once per chunk, before the row loop, which then
+        # takes them like inputs; the epilogue reuses them.
+        rfront = []
+        for g_ in (p.restep, p.drow):
+            for n_ in g_.nodes:
+                if not n_.ext[0] and n_.op != 'const' and n_.name not in rfront and \
+                        any(n_.name in m_.value_args() and m_.ext[0] for m_ in g_.nodes):
+                    rfront.append(n_.name)
+        cut_all = front + rfront
+        restep_g = p.restep.extract('restep', p.restep.outputs, cut=cut_all) if cut_all else p.restep
         drow_outs = list(p.drow.outputs[:nst + len(mats2)]) + [op_names[j] for j in loop_ops]
-        drow_g = p.drow.extract('drow', drow_outs, cut=front) if front else p.drow
+        drow_g = p.drow.extract('drow', drow_outs, cut=cut_all) if cut_all else p.drow
         drow_exts = st_ext + [(True, True)] * len(mats2) + [self.jext[op_names[j]] for j in loop_ops]
         drow_src, drow_used = emit_graph_fn(drow_g, 'bw_drow', 1, 1, drow_exts, red, self.invariant)
         re_src, re_used = emit_graph_fn(restep_g, 'bw_restep', 1, 1, st_ext, red, self.invariant)
         epi_exts = [self.in_ext(i) for i in rs]
-        epi_src, epi_used = emit_graph_fn(p.epi, 'bw_epi', 1, 1, epi_exts, red)
+        epi_nodes = {n_.name for n_ in p.epi.nodes}
+        epi_g = p.epi.extract('epi', p.epi.outputs, cut=[f for f in rfront if f in epi_nodes]) if rfront else p.epi
+        epi_src, epi_used = emit_graph_fn(epi_g, 'bw_epi', 1, 1, epi_exts, red)
         loop_used = set(drow_used) | set(re_used)
-        all_used = loop_used | set(epi_used)
         pre_src, pre_used = '', []
+        cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
         if front:
-            cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
             pre_g = p.joint.extract('colpre', front, cut=set(cuts))
             pre_src, pre_used = emit_graph_fn(pre_g, 'bw_colpre', 1, 1, [(True, False)] * len(front), red, self.invariant)
+        rpre_used = []
+        if rfront:
+            rpre_g = p.joint.extract('rowpre', rfront, cut=set(cuts))
+            rpre_src, rpre_used = emit_graph_fn(rpre_g, 'bw_rowpre', 1, 1, [self.jext[f] for f in rfront], red, self.invariant)
+            pre_src += '\n' + rpre_src
+        all_used = loop_used | set(epi_used) | set(rpre_used)
 
         def is_rowlike(nm):      # no row extent: can be loaded once per chunk
             return not self.jext[nm][0]
@@ -892,6 +998,19 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for j in loop_ops:
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
+        if rfront:
+            for tt in range(DT):
+                call = []
+                for v in rpre_used:
+                    if v in p.in_names:
+                        call.append(var_in(p.in_names.index(v), tt))
+                    else:
+                        assert v in p.aux and is_rowlike(v), v
+                        call.append(f'ax{p.aux.index(v)}_{tt}')
+                for q in range(len(rfront)):
+                    b.append(f'  float g{q}_{tt}[1][1];\n')
+                    call.append(f'g{q}_{tt}')
+                b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
         # ---- per-row operands of the chunk go through LDS: staged once per row block by the
         # instance's own lanes (coalesced along m), read back per row as broadcast vectors
         rowops = []          # (lds name, loader(tt, mexpr) -> expr, register prefix)
@@ -1014,6 +1133,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     call.append(f'ms{p.msums.index(v)}')
                 elif v in front:
                     call.append(f'f{front.index(v)}_{tt}')
+                elif v in rfront:
+                    call.append(f'g{rfront.index(v)}_{tt}')
                 else:
                     raise AssertionError(v)
             return call

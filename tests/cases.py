@@ -13,6 +13,7 @@ CASES = {
     'gla': (ops.gla, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('row', 'BTH')], 1),
     'retention': (ops.retention, [('scalar', 'BTH'), ('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH')], 1),
     'delta_rule': (ops.delta_rule, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('scalar', 'BTH')], 1),
+    'delta_rule_fused': (ops.delta_rule_fused, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('scalar', 'BTH')], 1),
     'gated_delta_rule': (ops.gated_delta_rule, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('scalar', 'BTH'), ('scalar', 'BTH')], 1),
     'mamba2': (ops.mamba2, [('col', 'BTH'), ('scalar', 'BTH'), ('scalar', 'H'), ('row', 'BT'), ('row', 'BT')], 1),
     'mamba': (ops.mamba, [('col', 'BTH'), ('col', 'BTH'), ('mat', 'H'), ('row', 'BT'), ('row', 'BT')], 1),

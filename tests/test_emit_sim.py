@@ -21,6 +21,8 @@ RUNS = [
     ('cfg:rwkv7', '1,16,2,128,128', 'bf16', 1),
     ('cfg:rwkv7', '1,16,2,128,128', 'f32', 0),
     ('cfg:gated_delta_rule', '1,16,2,128,128', 'bf16', 1),
+    ('rwkv7', '1,16,2,64,64', 'bf16', 0),           # log-decay: exp evaluated while staging / once per chunk
+    ('delta_rule_fused', '2,16,2,16,32', 'f32', 1), # in-step normalisation (row-only sum) and gate
     ('rwkv6', '2,8,2,16,16', 'f32', 1),             # time-independent row input
     ('s4d', '2,8,1,8,16', 'f32', 1),                # two states, four matrix inputs
     ('longhorn', '2,8,2,16,8', 'f32', 0),           # row-only forward sum
