@@ -180,9 +180,14 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
         C //= 2
         L, G, R, W, waves = geometry(C)
     MT = W * G * R
+    R1 = W1 = 0
     if part.dstep_needs_state:
-        # the reverse scan keeps the DT recomputed states of a chunk in registers
-        DT = max(2, min(16, _pow2_floor(128 // max(R * C * nst, 1))))
+        # the reverse scan keeps the DT recomputed states of a chunk in registers: one row per
+        # lane there, and a chunk short enough for 64 registers of history per state (measured:
+        # anything more drops the kernel to one wave per SIMD or spills)
+        R1 = 1
+        W1 = max(1, min(4, M // G)) if G <= M else 1
+        DT = max(2, min(16, _pow2_floor(64 // max(C * part.nstates, 1))))
     else:
         DT = 16
     while DT > 1 and DT > T:              # a partial last chunk is handled in the kernels
@@ -208,7 +213,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     if part.epi_linear:
         while waves2 * MS < 32 * 4 * n_cu and -(-M // (2 * MS)) >= 8:
             MS *= 2
-    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, HB=1, MS=MS)
+    return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, R1=R1, W1=W1, HB=1, MS=MS)
 
 
 def check_tile(tile: TileConfig, H: int, N: int, part: Partition) -> None:
