@@ -336,6 +336,13 @@ def _col_expr(C: int, L: int) -> str:
     return f'(l * {C} + (c))'
 
 
+def needs_gradient_kernel(part) -> bool:
+    """The per-chunk gradient kernel produces the row- and scalar-input gradients and, unless the
+    reverse scan already does, the matrix-input gradients.  A recurrence with none of these
+    (all inputs per-row, e.g. a vector state) is finished after the reverse scan."""
+    return bool(part.row_idx or part.scalar_idx or (part.mat_idx and not part.mat_in_dstep))
+
+
 class Emitter:
     def __init__(self, plan):
         self.plan = plan
@@ -664,8 +671,9 @@ class Emitter:
         body.append(stg.load('tlast', '  '))
         body.append(f'  for (int t0 = tlast; t0 >= 0; t0 -= {TS}) {{\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
+        # d_state checkpoints are only read by the gradient kernel
         body.append(f'    if ((t0 + {TS}) % {DT} == 0{f" || t0 + {TS} >= T" if self.tail_dt else ""}) {{\n')
-        for k in range(nst):
+        for k in range(nst if needs_gradient_kernel(p) else 0):
             rr, cc = _dims(st_ext[k], R, C)
             body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '

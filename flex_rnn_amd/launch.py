@@ -17,7 +17,7 @@ from typing import Dict, List, Sequence, Tuple
 import torch as th
 
 from . import runtime
-from .emit_hip import Emitter, KernelSpec
+from .emit_hip import Emitter, KernelSpec, needs_gradient_kernel
 
 
 def _strides5(t: th.Tensor) -> Tuple[int, ...]:
@@ -25,17 +25,9 @@ def _strides5(t: th.Tensor) -> Tuple[int, ...]:
     return tuple(s + [0] * (5 - len(s)))
 
 
-def needs_gradient_kernel(plan) -> bool:
-    """The per-chunk gradient kernel produces the row- and scalar-input gradients and, unless the
-    reverse scan already does, the matrix-input gradients.  A recurrence with none of these
-    (all inputs per-row, e.g. a vector state) is finished after the reverse scan."""
-    p = plan.part
-    return bool(p.row_idx or p.scalar_idx or (p.mat_idx and not p.mat_in_dstep))
-
-
 def kernel_specs(plan) -> List[KernelSpec]:
     em = Emitter(plan)
-    return [em.fw(), em.bw1()] + ([em.bw2()] if needs_gradient_kernel(plan) else [])
+    return [em.fw(), em.bw1()] + ([em.bw2()] if needs_gradient_kernel(plan.part) else [])
 
 
 MAX_SPILL_BYTES = 64      # per lane; beyond this a higher-occupancy build of the gradient kernel is not taken
@@ -155,7 +147,8 @@ class CompiledPlan:
         B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
         atomic = set(pl.atomic)
         daux = th.empty(len(p.daux), B, H, T, M, dtype=th.float32, device=dev)
-        dck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state_store)
+        dck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state_store) \
+            if 'frnn_bw2' in self.kernels else ()
         if self.state_meta is not None:
             dst0 = tuple(th.empty_strided(sh, st, dtype=dt, device=dev) for sh, st, dt in self.state_meta)
         else:
@@ -174,7 +167,8 @@ class CompiledPlan:
             tensors[f'dstT{k}'] = dstateT[k]
             tensors[f'dst{k}'] = dst0[k]
             tensors[f'sck{k}'] = state_store[k]
-            tensors[f'dck{k}'] = dck[k]
+            if dck:
+                tensors[f'dck{k}'] = dck[k]
         for k in range(p.noutputs):
             tensors[f'dout{k}'] = doutput[k]
         self._launch('frnn_bw1', tensors)

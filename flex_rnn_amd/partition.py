@@ -191,7 +191,10 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
     # backward sum reads it), it also accumulates the matrix-input gradients over the whole
     # sequence in registers; otherwise the gradient kernel does, chunk by chunk.
     probe = joint.extract('probe', list(dst_names) + [din_names[i] for i in col_idx], cut=set(aux_all))
-    mat_in_dstep = bool(mat_idx) and any(probe.uses(s_) for s_ in st_names)
+    # The same holds when the gradient kernel would have nothing else to do (no row or scalar
+    # input): recomputing the state in the reverse scan is cheaper than a kernel whose every
+    # chunk adds a full matrix of partial gradients with atomics.
+    mat_in_dstep = bool(mat_idx) and (any(probe.uses(s_) for s_ in st_names) or not (row_idx or scalar_idx))
     mats_drow = [] if mat_in_dstep else list(mat_idx)
     mats_dstep = list(mat_idx) if mat_in_dstep else []
 
