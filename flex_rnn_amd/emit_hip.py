@@ -113,6 +113,7 @@ _UNARY_EXPR = {
     'sqrt': 'sqrtf({0})', 'rsqrt': 'rsqrtf({0})', 'sigmoid': 'f_sigmoid({0})', 'tanh': 'f_tanh({0})',
     'abs': '__builtin_fabsf({0})', 'relu': 'fmaxf({0}, 0.0f)', 'sign': 'f_sign({0})',
     'log1p': 'log1pf({0})', 'expm1': 'expm1f({0})', 'copy': '({0})',
+    'sin': 'sinf({0})', 'cos': 'cosf({0})', 'erf': 'erff({0})', 'log2': '__log2f({0})', 'exp2': 'f_exp2({0})',
 }
 _BINARY_EXPR = {
     'mul': '({0} * {1})', 'add': '({0} + {1})', 'sub': '({0} - {1})', 'div': '({0} / {1})',

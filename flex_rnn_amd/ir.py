@@ -27,7 +27,7 @@ Arg = Union[str, float, int, bool]
 
 # op name -> arity.  Semantics are fp32; comparisons yield 0.0 / 1.0.
 UNARY_OPS = ('exp', 'neg', 'reciprocal', 'log', 'sqrt', 'rsqrt', 'sigmoid', 'tanh', 'abs',
-             'relu', 'sign', 'log1p', 'expm1', 'copy')
+             'relu', 'sign', 'log1p', 'expm1', 'copy', 'sin', 'cos', 'erf', 'log2', 'exp2')
 BINARY_OPS = ('mul', 'add', 'sub', 'div', 'lt', 'gt', 'le', 'ge', 'eq', 'ne', 'maximum', 'minimum')
 TERNARY_OPS = ('where',)
 ALL_OPS = UNARY_OPS + BINARY_OPS + TERNARY_OPS + ('sum', 'const')

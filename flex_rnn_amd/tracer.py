@@ -95,7 +95,8 @@ _ALIAS = {'aten::_to_copy', 'aten::clone', 'aten::expand', 'aten::alias', 'aten:
 _UNARY = {'aten::exp': 'exp', 'aten::neg': 'neg', 'aten::reciprocal': 'reciprocal', 'aten::log': 'log',
           'aten::sqrt': 'sqrt', 'aten::rsqrt': 'rsqrt', 'aten::sigmoid': 'sigmoid', 'aten::tanh': 'tanh',
           'aten::abs': 'abs', 'aten::relu': 'relu', 'aten::sign': 'sign', 'aten::sgn': 'sign',
-          'aten::log1p': 'log1p', 'aten::expm1': 'expm1'}
+          'aten::log1p': 'log1p', 'aten::expm1': 'expm1', 'aten::sin': 'sin', 'aten::cos': 'cos',
+          'aten::erf': 'erf', 'aten::log2': 'log2', 'aten::exp2': 'exp2'}
 _BINARY = {'aten::mul': 'mul', 'aten::add': 'add', 'aten::sub': 'sub', 'aten::div': 'div', 'aten::lt': 'lt',
            'aten::gt': 'gt', 'aten::le': 'le', 'aten::ge': 'ge', 'aten::eq': 'eq', 'aten::ne': 'ne',
            'aten::maximum': 'maximum', 'aten::minimum': 'minimum'}
@@ -222,8 +223,13 @@ def fx_to_graph(gm: torch.fx.GraphModule, name: str = 'joint') -> Graph:
                 env[node.name] = b.emit('rsqrt', (x,), hint='rsqrt')
             elif p == 0.0:
                 env[node.name] = b.const(1.0)
-            else:
-                raise UnsupportedOp(f'pow with exponent {p} is not supported')
+            elif p == int(p) and abs(p) <= 8:
+                r = x
+                for _ in range(int(abs(p)) - 1):
+                    r = b.emit('mul', (r, x), hint='mul')
+                env[node.name] = r if p > 0 else b.emit('reciprocal', (r,), hint='reciprocal')
+            else:       # positive bases only, like torch for a fractional exponent
+                env[node.name] = b.emit('exp', (b.emit('mul', (b.emit('log', (x,), hint='log'), p), hint='mul'),), hint='exp')
         elif base == 'aten::where':
             env[node.name] = b.emit('where', (lift(a[0]), lift(a[1]), lift(a[2])), hint='where')
         elif base in _CONST_LIKE:
@@ -262,6 +268,74 @@ def fx_to_graph(gm: torch.fx.GraphModule, name: str = 'joint') -> Graph:
             if scale != 1:
                 r = b.emit('mul', (r, float(scale)), hint='mul')
             env[node.name] = r
+        elif base in ('aten::clamp', 'aten::hardtanh', 'aten::clamp_min', 'aten::clamp_max'):
+            r = lift(a[0])
+            if base == 'aten::hardtanh':
+                lo, hi = (a[1] if len(a) > 1 else kw.get('min_val', -1.0)), (a[2] if len(a) > 2 else kw.get('max_val', 1.0))
+            elif base == 'aten::clamp_min':
+                lo, hi = a[1], None
+            elif base == 'aten::clamp_max':
+                lo, hi = None, a[1]
+            else:
+                lo, hi = (a[1] if len(a) > 1 else kw.get('min')), (a[2] if len(a) > 2 else kw.get('max'))
+            if lo is not None:
+                r = b.emit('maximum', (r, val(lo)), hint='maximum')
+            if hi is not None:
+                r = b.emit('minimum', (r, val(hi)), hint='minimum')
+            env[node.name] = r
+        elif base == 'aten::hardtanh_backward':
+            g, x = lift(a[0]), lift(a[1])
+            inside = b.emit('mul', (b.emit('gt', (x, float(a[2])), hint='gt'), b.emit('lt', (x, float(a[3])), hint='lt')), hint='mul')
+            env[node.name] = b.emit('mul', (g, inside), hint='mul')
+        elif base in ('aten::logical_and', 'aten::bitwise_and', 'aten::logical_or', 'aten::bitwise_or'):
+            # truth values are 0.0 / 1.0 floats here
+            x, y = (b.emit('ne', (lift(v), 0.0), hint='ne') for v in a[:2])
+            env[node.name] = b.emit('mul' if base.endswith('and') else 'maximum', (x, y), hint='and' if base.endswith('and') else 'or')
+        elif base in ('aten::logical_not', 'aten::bitwise_not'):
+            env[node.name] = b.emit('eq', (lift(a[0]), 0.0), hint='not')
+        elif base == 'aten::leaky_relu':
+            x, slope = lift(a[0]), float(a[1] if len(a) > 1 else kw.get('negative_slope', 0.01))
+            env[node.name] = b.emit('where', (b.emit('gt', (x, 0.0), hint='gt'), x, b.emit('mul', (x, slope), hint='mul')), hint='where')
+        elif base == 'aten::leaky_relu_backward':
+            g, x, slope = lift(a[0]), lift(a[1]), float(a[2])
+            env[node.name] = b.emit('where', (b.emit('gt', (x, 0.0), hint='gt'), g, b.emit('mul', (g, slope), hint='mul')), hint='where')
+        elif base == 'aten::elu':
+            x = lift(a[0])
+            alpha, scale, iscale = (float(a[i]) if len(a) > i else 1.0 for i in (1, 2, 3))
+            neg = b.emit('mul', (b.emit('expm1', (b.emit('mul', (x, iscale), hint='mul'),), hint='expm1'), alpha * scale), hint='mul')
+            env[node.name] = b.emit('where', (b.emit('gt', (x, 0.0), hint='gt'), b.emit('mul', (x, scale), hint='mul'), neg), hint='where')
+        elif base == 'aten::elu_backward':
+            g, alpha, scale, iscale, is_result, x = lift(a[0]), float(a[1]), float(a[2]), float(a[3]), bool(a[4]), lift(a[5])
+            if is_result:
+                neg = b.emit('mul', (g, b.emit('mul', (b.emit('add', (x, alpha * scale), hint='add'), iscale), hint='mul')), hint='mul')
+            else:
+                e = b.emit('exp', (b.emit('mul', (x, iscale), hint='mul'),), hint='exp')
+                neg = b.emit('mul', (g, b.emit('mul', (e, alpha * scale * iscale), hint='mul')), hint='mul')
+            env[node.name] = b.emit('where', (b.emit('gt', (x, 0.0), hint='gt'), b.emit('mul', (g, scale), hint='mul'), neg), hint='where')
+        elif base in ('aten::gelu', 'aten::gelu_backward'):
+            bw = base.endswith('backward')
+            g = lift(a[0]) if bw else None
+            x = lift(a[1] if bw else a[0])
+            approx = kw.get('approximate', a[2 if bw else 1] if len(a) > (2 if bw else 1) else 'none')
+            mul = lambda u, v: b.emit('mul', (u, v), hint='mul')
+            add = lambda u, v: b.emit('add', (u, v), hint='add')
+            if approx == 'tanh':
+                k, c = 0.7978845608028654, 0.044715
+                x2 = mul(x, x)
+                t = b.emit('tanh', (mul(mul(x, add(mul(x2, c), 1.0)), k),), hint='tanh')
+                cdf = mul(add(t, 1.0), 0.5)
+                if not bw:
+                    env[node.name] = mul(x, cdf)
+                else:
+                    dt = mul(b.emit('sub', (b.const(1.0), mul(t, t)), hint='sub'), mul(add(mul(x2, 3.0 * c), 1.0), k))
+                    env[node.name] = mul(g, add(cdf, mul(mul(x, 0.5), dt)))
+            else:
+                cdf = mul(add(b.emit('erf', (mul(x, 0.7071067811865476),), hint='erf'), 1.0), 0.5)
+                if not bw:
+                    env[node.name] = mul(x, cdf)
+                else:
+                    pdf = mul(b.emit('exp', (mul(mul(x, x), -0.5),), hint='exp'), 0.3989422804014327)
+                    env[node.name] = mul(g, add(cdf, mul(x, pdf)))
         elif base == 'aten::sigmoid_backward':
             g, out = lift(a[0]), lift(a[1])
             t = b.emit('sub', (b.const(1.0), out), hint='sub')

@@ -23,7 +23,8 @@ _UN = {
     'exp': torch.exp, 'neg': torch.neg, 'reciprocal': torch.reciprocal, 'log': torch.log,
     'sqrt': torch.sqrt, 'rsqrt': torch.rsqrt, 'sigmoid': torch.sigmoid, 'tanh': torch.tanh,
     'abs': torch.abs, 'relu': torch.relu, 'sign': torch.sign, 'log1p': torch.log1p,
-    'expm1': torch.expm1, 'copy': lambda x: x,
+    'expm1': torch.expm1, 'copy': lambda x: x, 'sin': torch.sin, 'cos': torch.cos, 'erf': torch.erf,
+    'log2': torch.log2, 'exp2': torch.exp2,
 }
 _BIN = {
     'mul': torch.mul, 'add': torch.add, 'sub': torch.sub, 'div': torch.div,

@@ -37,6 +37,23 @@ def _zoo(x, g, c, S):
 
 CASES['zoo'] = (_zoo, [('row', 'BTH'), ('row', 'BT'), ('col', 'BTH')], 1)
 
+
+def _zoo2(x, g, c, S):
+    """More of the op table: clamp / hardtanh, leaky_relu, elu, gelu (both forms), silu, sin, cos, erf,
+    log2, exp2, integer and fractional powers, logical and / or / not on comparisons."""
+    gate = th.sigmoid(F.gelu(g) + F.gelu(x, approximate='tanh') * 0.5 + F.silu(g) * 0.1)
+    upd = F.leaky_relu(x, 0.1) + F.elu(x) * 0.3 + x.clamp(-0.7, 0.9) + F.hardtanh(g, -0.5, 0.5) + g.clamp(min=-0.2) * 0.1
+    upd = upd + th.sin(x) * th.cos(g) + th.erf(x) * 0.2 + th.log2(1.5 + x * x) * th.exp2(-g.abs())
+    upd = upd + (x.abs() + 0.5) ** 1.5 * 0.1 + (0.5 * x) ** 4 + (1.0 + g * g) ** -2
+    inside = (x > -0.3) & (x < 0.6)
+    outside = (g > 1.0) | ~(g > -1.0)
+    S = S * gate + c * th.where(inside, upd, 0.5 * upd) + th.where(outside, g, x) * 0.05 * F.relu6(c + 1.0)
+    y = (S * th.tanh(x)).sum(-1, True) + F.hardsigmoid(c) * F.hardswish(c) * 0.1
+    return y, S
+
+
+CASES['zoo2'] = (_zoo2, [('row', 'BTH'), ('row', 'BT'), ('col', 'BTH')], 1)
+
 # vector-state recurrences (N == 1)
 VECTOR_CASES = {
     'hgrn': (ops.hgrn, [('col', 'BT'), ('col', 'BT')], 1),
@@ -79,3 +96,62 @@ def make_inputs(name, B, T, H, M, N, dtype=th.float64, seed=0, table=None):
     Heff = H if any('H' in spans for _, spans in spec) else 1      # states follow the widest input
     ss = [(th.randn(B, Heff, M, N, generator=g) * 0.3).to(dtype) for _ in range(nst)]
     return step, xs, ss
+
+
+# ------------------------------------------------------------------ random recurrences
+_UNARY_SRC = ['th.sigmoid({0})', 'th.tanh({0})', '({0}).exp().clamp(max=4.0)', 'F.softplus({0})', '({0} * {0})',
+              '(1.0 / (1.0 + ({0}).abs()))', 'th.where({0} > 0, {0}, 0.3 * {0})', '(-{0})', '({0} * 0.5 + 0.1)']
+
+
+def random_step(seed):
+    """A random but well-behaved linear-attention-like recurrence: a contractive decay built from
+    a random mix of row / column / scalar inputs, one or two rank-1 updates, optionally a
+    delta-rule style read-back (S k) and an in-step normalisation, and a read-out with an
+    optional per-row skip term.  Returns (step, spec, nstates, source)."""
+    import random
+    rnd = random.Random(seed)
+    ninp = rnd.randint(3, 6)
+    classes = ['row', 'col'] + [rnd.choice(['row', 'col', 'scalar', 'row']) for _ in range(ninp - 2)]
+    rnd.shuffle(classes)
+    spec = []
+    for c in classes:
+        spans = ''.join(d for d in 'BTH' if rnd.random() < 0.8)
+        spec.append((c, spans))
+    spec[0] = (spec[0][0], 'BTH')
+    names = [f'x{i}' for i in range(ninp)]
+    by = {c: [n for n, (cc, _) in zip(names, spec) if cc == c] for c in ('row', 'col', 'scalar')}
+
+    def pick(cls_list):
+        pool = [n for c in cls_list for n in by[c]]
+        return rnd.choice(pool)
+
+    def expr(cls_list, depth=2):
+        e = pick(cls_list)
+        for _ in range(rnd.randint(0, depth)):
+            e = rnd.choice(_UNARY_SRC).format(e)
+            if rnd.random() < 0.3:
+                e = f'({e} * {pick(cls_list)})'
+        return e
+
+    lines = []
+    if rnd.random() < 0.4:          # in-step normalisation of a row input
+        r0 = by['row'][0]
+        lines.append(f'{r0} = {r0} * th.rsqrt(({r0} * {r0}).sum(-1, True) + 1.0)')
+    dec = [rnd.choice([['row'], ['col'], ['row', 'scalar'] if by['scalar'] else ['row'], ['col', 'row']])]
+    lines.append(f'decay = th.sigmoid({expr(dec[0])})' + (f' * th.sigmoid({expr(["col"])})' if rnd.random() < 0.4 else ''))
+    lines.append(f'k = {expr(["row", "scalar"] if by["scalar"] else ["row"])}')
+    lines.append(f'v = {expr(["col", "scalar"] if by["scalar"] else ["col"])}')
+    if rnd.random() < 0.5:          # delta-rule style correction
+        lines.append('S = S * decay')
+        lines.append(f'S = S + 0.5 * th.sigmoid({pick(["row", "col", "scalar"] if by["scalar"] else ["row", "col"])}) * k * (v - (S * k).sum(-1, True))')
+    else:
+        lines.append('S = S * decay + v * k')
+        if rnd.random() < 0.5:
+            lines.append(f'S = S + 0.1 * (S * th.tanh({expr(["row"])})).sum(-1, True) * th.tanh({expr(["row"])})')
+    lines.append(f'y = (S * {expr(["row"])}).sum(-1, True)')
+    if rnd.random() < 0.5:
+        lines.append(f'y = y + {expr(["col"])}')
+    src = 'def step(' + ', '.join(names) + ', S):\n' + ''.join(f'    {ln}\n' for ln in lines) + '    return y, S\n'
+    env = {'th': th, 'F': F}
+    exec(src, env)
+    return env['step'], spec, 1, src

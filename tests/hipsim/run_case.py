@@ -32,6 +32,10 @@ def main():
         table = {'pat': (step, [(c, sp) for c, sp in spec], 1)}
         step, xs, ss = cases.make_inputs('pat', *dims, dtype=dtype, table=table)
         ss = [th.randn(dims[0], dims[2], dims[3], dims[4], generator=th.Generator().manual_seed(3)).to(dtype) * 0.3]
+    elif name.startswith('gen:'):
+        step, spec, nst, src = cases.random_step(int(name[4:]))
+        print(src)
+        step, xs, ss = cases.make_inputs('gen', *dims, dtype=dtype, table={'gen': (step, spec, nst)})
     elif name.startswith('cfg:'):
         wl = configs.make(name[4:], dims=dims, dtype=dtype)
         step, xs, ss = wl.step, wl.inputs, wl.states

@@ -39,6 +39,7 @@ RUNS = [
     ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1),
     # the emitter's op table (sigmoid, tanh, softplus, where, relu, sqrt, rsqrt, log, min/max, ...)
     ('zoo', '2,8,2,16,16', 'f32', 1),
+    ('zoo2', '2,8,2,16,16', 'f32', 0),
     # state heights that are not a power of two (row masking), fp64 and fp16 I/O
     ('cfg:rwkv7', '1,16,1,24,128', 'f32', 0),
     ('gla', '2,8,2,100,32', 'f32', 1),
@@ -94,3 +95,11 @@ def test_random_broadcast_patterns(seed):
     case = _random_pattern_case(seed)
     r = subprocess.run([sys.executable, RUNNER, case, '2,8,3,8,16', 'f32', str(seed % 2)], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'{case}\nrc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
+
+
+@pytest.mark.parametrize('seed', range(100, 112))
+def test_random_recurrences(seed):
+    """Random step functions (tests/cases.py: random_step) through the emitted kernels."""
+    dims = ['2,8,2,8,16', '1,19,2,5,32', '2,16,1,24,128'][seed % 3]
+    r = subprocess.run([sys.executable, RUNNER, f'gen:{seed}', dims, 'f32', str(seed % 2), '1e-4'], capture_output=True, text=True, timeout=900)
+    assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2500:]}\n{r.stderr[-3000:]}'

@@ -177,7 +177,7 @@ def test_check_grad_and_benchmark_helpers():
 @pytest.mark.parametrize('name,dims', [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn', (2, 32, 2, 32, 16)),
                                        ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
                                        ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)),
-                                       ('zoo', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
+                                       ('zoo', (2, 32, 2, 32, 32)), ('zoo2', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
                                        # pointwise preparation inside the step: log-decay, in-step normalisation
                                        ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32))])
 def test_other_recurrences(name, dims):

@@ -41,6 +41,29 @@ def test_partition_single_row_state(name, M, N):
     _check(name, 2, 8, 2, M, N, DT=4)
 
 
+@pytest.mark.parametrize('seed', range(40))
+def test_partition_of_random_recurrences(seed):
+    """Random step functions (tests/cases.py: random_step): whatever the partition accepts must
+    reproduce autograd of the plain loop; a rejection must be a named PartitionError."""
+    from flex_rnn_amd.partition import PartitionError
+    step, spec, nst, src = cases.random_step(seed)
+    table = {'gen': (step, spec, nst)}
+    step, xs, ss = cases.make_inputs('gen', 2, 8, 2, 4, 8, table=table)
+    try:
+        plan, _, _ = planner.make_plan(step, xs, ss)
+    except PartitionError:
+        return
+    g = th.Generator().manual_seed(5)
+    out = recurrence.run_loop(step, xs, ss)
+    dy = [th.randn(o.shape, generator=g, dtype=th.float64) for o in out[0]]
+    dS = [th.randn(s_.shape, generator=g, dtype=th.float64) for s_ in ss]
+    want = recurrence.loop_with_grads(step, xs, ss, dy, dS)
+    got = plan_exec.run_plan(plan.part, xs, ss, dy, dS, DT=4)
+    for a, b in zip(got, want):
+        for x, y in zip(a, b):
+            assert x.shape == y.shape and recurrence.rel_err(x, y) < 1e-9, src
+
+
 def test_aux_daux_of_rwkv7():
     plan = _check('rwkv7_decay', 1, 4, 1, 4, 4, DT=2)
     p = plan.part

@@ -17,7 +17,7 @@ OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn'
          ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
          ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)), ('gla', (1, 16, 1, 16, 16)),
          ('gla', (1, 32, 1, 16, 16)), ('delta_rule', (2, 32, 2, 16, 16)), ('gated_delta_rule', (2, 32, 2, 16, 16)),
-         ('zoo', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
+         ('zoo', (2, 32, 2, 32, 32)), ('zoo2', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
          ('gla', (1, 16, 2, 16, 16)), ('gla', (3, 50, 2, 16, 16)), ('gla', (2, 33, 2, 16, 16)),
          ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32))]
 
