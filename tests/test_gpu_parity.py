@@ -42,3 +42,28 @@ def test_parity_reduced(name, dims, dtype):
     tol = TOL[wl.dtype]
     print('rel errors', ['%.2e' % e for e in errs], flush=True)
     assert max(errs) < tol, (name, errs)
+
+
+@pytest.mark.parametrize('name', ['delta_rule', 'mamba1', 'mamba2', 'rwkv7', 'gated_delta_rule'])
+def test_committed_vectors(name):
+    """The compiled path on the inputs of tests/golden/five_configs_fp64.npz (fp32 I/O) against the
+    stored fp64 results: <= 1e-4."""
+    import os
+    import numpy as np
+    print(f'case golden {name}', flush=True)
+    z = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'five_configs_fp64.npz'))
+
+    def arrs(key):
+        out, i = [], 0
+        while f'{name}.{key}{i}' in z:
+            out.append(th.from_numpy(z[f'{name}.{key}{i}']))
+            i += 1
+        return out
+    step = configs.make(name, dims=(1, 2, 1, 2, 2), dtype=th.float32).step
+    xs = [x.float().cuda().requires_grad_() for x in arrs('in')]
+    ss = [s.float().cuda().requires_grad_() for s in arrs('st')]
+    res = flex_rnn_amd.jit(step)(*xs, *ss)
+    grads = th.autograd.grad(res, xs + ss, [g.float().cuda() for g in arrs('dy') + arrs('dS')])
+    want = arrs('out') + arrs('stT') + arrs('din') + arrs('dst')
+    errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
+    assert max(errs) < 1e-4, errs

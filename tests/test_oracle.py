@@ -158,3 +158,30 @@ def test_package_naive_matches_oracle(dtype):
     assert y64.dtype == th.float64
     (y64o,), _ = recurrence.run_loop(ops.rwkv7_decay, xs, ss, dtype=th.float64)
     assert recurrence.rel_err(y64, y64o) == 0
+
+
+@pytest.mark.parametrize('name', ['delta_rule', 'mamba1', 'mamba2', 'rwkv7', 'gated_delta_rule'])
+def test_committed_vectors(name):
+    """tests/golden/five_configs_fp64.npz (written by tests/golden/make_vectors.py from this oracle) is
+    a fixed point: the oracle, the package's `naive` and the step functions still give those numbers."""
+    import os
+    import numpy as np
+    import flex_rnn_amd
+    from flex_rnn_amd import configs
+    z = np.load(os.path.join(os.path.dirname(__file__), 'golden', 'five_configs_fp64.npz'))
+
+    def arrs(key):
+        out, i = [], 0
+        while f'{name}.{key}{i}' in z:
+            out.append(th.from_numpy(z[f'{name}.{key}{i}']))
+            i += 1
+        return out
+    step = configs.make(name, dims=(1, 2, 1, 2, 2), dtype=th.float64).step
+    xs, ss, dy, dS = arrs('in'), arrs('st'), arrs('dy'), arrs('dS')
+    res = recurrence.loop_with_grads(step, xs, ss, dy, dS)
+    for key, got in zip(('out', 'stT', 'din', 'dst'), res):
+        for a, b in zip(got, arrs(key)):
+            assert a.shape == b.shape and recurrence.rel_err(a, b) < 1e-12, (name, key)
+    naive = flex_rnn_amd.jit(step).naive(*xs, *ss, dtype=th.float64)
+    for a, b in zip(naive, arrs('out') + arrs('stT')):
+        assert recurrence.rel_err(a, b) < 1e-12

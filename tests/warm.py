@@ -52,6 +52,10 @@ def warm_examples(force=False, seen=None):
     return n
 
 
+GOLDEN = {'delta_rule': (1, 6, 2, 4, 4), 'mamba1': (2, 6, 2, 4, 4), 'mamba2': (2, 6, 2, 4, 8),
+          'rwkv7': (2, 6, 2, 4, 8), 'gated_delta_rule': (2, 6, 2, 4, 8)}      # tests/golden/make_vectors.py
+
+
 def warm(force=False, seen=None):
     n = warm_examples(force, seen)
     for name, dims in OTHER:
@@ -62,6 +66,8 @@ def warm(force=False, seen=None):
         step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
         n += len(compile_plan(plan, force=force, seen=seen))
+    for name, dims in GOLDEN.items():
+        n += len(compile_plan(prebuild.plan_for(name, dims, th.float32), force=force, seen=seen))
     for name in ('rwkv7', 'gated_delta_rule'):
         B, T, H, M, N = configs.DEFAULT_DIMS[name]
         n += len(compile_plan(prebuild.plan_for(name, (B, 128, H, M, N)), force=force, seen=seen))
