@@ -90,34 +90,38 @@ class CompiledPlan:
                 kern = mod.kernel(spec.name)
             self.modules.append(mod)
             self.kernels[spec.name] = (spec, kern)
+        # per kernel: grid (fixed by the plan's sizes) and one packer for the whole argument block
+        env = dict(B=plan.B, T=plan.T, H=plan.H, M=plan.M, nch=plan.nchunks)
+        self._grid = {k: tuple(int(eval(g, {}, env)) for g in s.grid) for k, (s, _) in self.kernels.items()}
+        self._packer = {k: struct.Struct('<' + 'q5q' * max(len(s.tensors), 1) + '5q') for k, (s, _) in self.kernels.items()}
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
         spec, kern = self.kernels[kname]
         pl = self.plan
-        buf = bytearray()
+        vals = []
         dev = None
         for name in spec.tensors:
             t = tensors[name]
             assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
             dev = t.device if dev is None else dev
             assert t.device == dev, 'all tensors must live on the same device'
-            buf += struct.pack('<q5q', t.data_ptr(), *_strides5(t))
+            vals.append(t.data_ptr())
+            vals.extend(_strides5(t))
         if not spec.tensors:
-            buf += struct.pack('<q5q', 0, 0, 0, 0, 0, 0)
-        buf += struct.pack('<5q', pl.B, pl.T, pl.H, pl.M, pl.nchunks)
-        env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
-        grid = tuple(int(eval(g, {}, env)) for g in spec.grid)
+            vals = [0] * 6
+        buf = self._packer[kname].pack(*vals, pl.B, pl.T, pl.H, pl.M, pl.nchunks)
+        grid = self._grid[kname]
         with th.cuda.device(dev):
             stream = th.cuda.current_stream(dev).cuda_stream
             if self.profile_events is not None:
                 e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
                 e0.record()
-                kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
+                kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
                 e1.record()
                 self.profile_events.append((kname, e0, e1))
             else:
-                kern.launch(grid, (spec.block, 1, 1), bytes(buf), stream=stream)
+                kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
 
     # ------------------------------------------------------------------ forward
     def forward(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
