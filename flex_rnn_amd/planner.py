@@ -150,6 +150,11 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     assert _is_pow2(N), f'state width N={N} must be a power of two (the state height M may be any size)'
     nst = part.nstates + len(part.mat_idx)
 
+    n_row = sum(1 for i in part.row_idx if in_bcast is None or not in_bcast[i][1])
+    r_lds = 1
+    while r_lds * 5 < 4 * n_row:
+        r_lds *= 2
+
     def geometry(C_):
         L_ = N // C_
         G_ = 64 // L_
@@ -165,8 +170,13 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
             w = waves_per_wg(r)
             return B * H * max(1, -(-M // (w * G_ * r))) * w
 
-        # ... and small enough that every SIMD holds at least two waves (latency hiding)
+        # ... and small enough that every SIMD holds at least two waves (latency hiding) ...
         while R_ > 1 and total_waves(R_) < 2 * 4 * n_cu:
+            R_ //= 2
+        # ... four, where LDS bandwidth allows: every lane reads C values of each staged row
+        # operand per step whatever R is, so fewer rows per lane means more LDS traffic per
+        # element (measured: 5 row operands at R = 4 keep the LDS half busy)
+        while R_ > r_lds and R_ // 2 >= r_lds and total_waves(R_) < 4 * 4 * n_cu:
             R_ //= 2
         return L_, G_, R_, waves_per_wg(R_), total_waves(R_)
 
