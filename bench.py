@@ -138,6 +138,11 @@ def main():
         'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
         'roofline': roofline, 'cpu_baseline': cpu,
         'gpu_kernel_ms_per_step': round(gpu_ms, 4),
+        # candidate builds of the gradient kernel as timed on the first backward call (the fastest runs)
+        'gradient_kernel_builds': [
+            {'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
+             'ms': compiled.bw2_times and round(compiled.bw2_times[i], 4)}
+            for i, (_, _, r) in enumerate(compiled.bw2_builds)],
         'forward_only': {'ms_per_step': round(fwd_ms, 4), 'tokens_per_s': round(tokens / (fwd_ms * 1e-3), 1),
                          'achieved_TFLOPs': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12, 3),
                          'frac': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4)},

@@ -830,7 +830,7 @@ class Emitter:
         return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
 
     # ------------------------------------------------------------------ bw2
-    def bw2(self, waves_per_simd: int = 0) -> KernelSpec:
+    def bw2(self, waves_per_simd: int = 0, prefetch: int = 4) -> KernelSpec:
         """`waves_per_simd` > 0 asks the compiler to fit that many waves on a SIMD (fewer registers,
         possibly spills); the caller compares the outcomes."""
         p, plan, t = self.p, self.plan, self.tile
@@ -840,7 +840,7 @@ class Emitter:
         HB = max(1, getattr(t, 'HB', 1))
         MS = max(1, getattr(t, 'MS', 1))
         MR = -(-plan.M // MS)               # rows per instance
-        PD = 4                              # checkpoint rows in flight ahead of the row loop
+        PD = max(1, prefetch)               # checkpoint rows in flight ahead of the row loop
         assert plan.H % HB == 0
         A = _Args()
         nin, nst, nout = p.ninputs, p.nstates, p.noutputs
@@ -1059,6 +1059,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         while MB * 2 <= MR and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
             MB *= 2
         lanes = min(N, NT)          # lanes of one instance
+        PDe = min(PD, MB)           # (a row block is a whole number of prefetch rounds)
         for nm_lds, _, _ in rowops:
             b.append(f'  __shared__ float {nm_lds}[{IPB}][{MB}][{DT}];\n')
 
@@ -1066,7 +1067,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for k in range(nst):
             b.append(f'  const float* sckp{k} = (const float*){A.p(f"sck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
             b.append(f'  const float* dckp{k} = (const float*){A.p(f"dck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
-            for j in range(PD):
+            for j in range(PDe):
                 b.append(f'  float Sq{k}_{j} = sckp{k}[min(mlo + {j}, M - 1) * {N}];\n  float Dq{k}_{j} = dckp{k}[min(mlo + {j}, M - 1) * {N}];\n')
         b.append(f'  for (int m0 = mlo; m0 < mhi; m0 += {MB}) {{\n')
         if rowops:
@@ -1099,18 +1100,18 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     q = front.index(op_names[j])
                     b.append(f'      {{ float a_ = 0.0f; for (int mm_ = 0; mm_ < nv_; mm_++) a_ += s_f{q}[inst][mm_][tt_]; s_cs{j}[inst][tt_] += a_; }}\n')
                 b.append('    }\n')
-        b.append(f'#pragma unroll {min(PD, MB)}\n  for (int mm = 0; mm < {MB}; mm++) {{\n    const int m = m0 + mm;\n    if (m >= mhi) break;\n')
+        # The row loop body is written out PDe times per iteration; copy j works on the row in
+        # slot j of a ring of checkpoint rows and refills that slot with the row PDe further on
+        # (fetched that many rows ahead of use: one row of arithmetic is shorter than a trip to HBM).
+        b.append(f'  for (int mm0 = 0; mm0 < {MB}; mm0 += {PDe}) {{\n')
+        body_start = len(b)
         for k in range(nst):
-            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Sq{k}_0;\n')
-            b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dq{k}_0;\n')
-        # checkpoint rows are fetched PD rows ahead of their use: one row of arithmetic is shorter
-        # than a trip to HBM
-        b.append(f'    {{ const int mn_ = min(m + {PD}, M - 1);\n')
+            b.append(f'    float Sh{k}_0[1][1]; Sh{k}_0[0][0] = Sq{k}_@J@;\n')
+            b.append(f'    float D{k}[1][1]; D{k}[0][0] = Dq{k}_@J@;\n')
+        b.append(f'    {{ const int mn_ = min(m + {PDe}, M - 1);\n')
         for k in range(nst):
-            for j in range(PD - 1):
-                b.append(f'      Sq{k}_{j} = Sq{k}_{j + 1}; Dq{k}_{j} = Dq{k}_{j + 1};\n')
-            b.append(f'      Sq{k}_{PD - 1} = sckp{k}[mn_ * {N}];\n')
-            b.append(f'      Dq{k}_{PD - 1} = dckp{k}[mn_ * {N}];\n')
+            b.append(f'      Sq{k}_@J@ = sckp{k}[mn_ * {N}];\n')
+            b.append(f'      Dq{k}_@J@ = dckp{k}[mn_ * {N}];\n')
         b.append('    }\n')
         for nm_lds, ld, pref in rowops:
             if ld is None and front[int(pref[1:])] not in loop_used:
@@ -1179,6 +1180,11 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             nmv = f'din{i}'
             idx = f'(i64)b * {A.s(nmv, 0)} + (i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)} + (i64)n * {A.s(nmv, 4)}'
             b.append(f'    if (valid) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
+        body = ''.join(b[body_start:])
+        del b[body_start:]
+        for j in range(PDe):
+            b.append(f'  {{\n    const int mm = mm0 + {j}; const int m = m0 + mm;\n    if (m >= mhi) break;\n'
+                     + body.replace('@J@', str(j)) + '  }\n')
         b.append('  }\n  }\n')
         # ---- epilogue
         def out_index(i, tt, hexpr):

@@ -10,6 +10,7 @@ fp32 scratch + cast-back for gradients of inputs broadcast over batch / time / h
 """
 from __future__ import annotations
 
+import os
 import struct
 from concurrent.futures import ThreadPoolExecutor
 from typing import Dict, List, Sequence, Tuple
@@ -25,59 +26,94 @@ def _strides5(t: th.Tensor) -> Tuple[int, ...]:
     return tuple(s + [0] * (5 - len(s)))
 
 
-def kernel_specs(plan) -> List[KernelSpec]:
+def kernel_specs(plan, prefetch: int = 4) -> List[KernelSpec]:
     em = Emitter(plan)
-    return [em.fw(), em.bw1()] + ([em.bw2()] if needs_gradient_kernel(plan.part) else [])
+    return [em.fw(), em.bw1()] + ([em.bw2(prefetch=prefetch)] if needs_gradient_kernel(plan.part) else [])
 
 
-MAX_SPILL_BYTES = 64      # per lane; beyond this a higher-occupancy build of the gradient kernel is not taken
+MAX_SPILL_BYTES = 64      # per lane; the untimed choice among gradient-kernel builds does not accept more
+
+
+def _compile(specs, force, seen):
+    jobs = []
+    for s in specs:
+        key = runtime.source_key(s.name, s.source)
+        again = force and (seen is None or key not in seen)
+        if seen is not None:
+            seen.add(key)
+        jobs.append((s, again))
+    # independent compiler processes: wait for them side by side (the runtime call releases the GIL)
+    with ThreadPoolExecutor(max_workers=max(1, len(jobs))) as pool:
+        paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
+    return [(s, path) for (s, _), path in zip(jobs, paths)]
+
+
+def gradient_kernel_builds(plan, force: bool = False, seen=None):
+    """Candidate builds of the gradient kernel, best guess first: [(spec, path, resources)].
+
+    The kernel is register-hungry (a chunk of accumulators per lane; RWKV-7 sits a few registers
+    below the limit for two waves per SIMD) and hides memory latency only through the waves
+    resident on its SIMD, so small changes of the generated code move it across occupancy
+    cliffs.  Builds with 4 and 2 checkpoint rows in flight are made, each also with a request
+    for one more wave per SIMD when that looks feasible.  Without a timing the order is decided
+    by the compiler's resource report: at most `MAX_SPILL_BYTES` spilled per lane, then more
+    waves per SIMD, then fewer spills, then the deeper prefetch.  `CompiledPlan` times them on
+    the first backward call and keeps the fastest."""
+    em = Emitter(plan)
+    cands, seen_src = [], set()
+
+    def add(spec):
+        if spec.source in seen_src:
+            return None
+        seen_src.add(spec.source)
+        path = _compile([spec], force, seen)[0][1]
+        res = runtime.kernel_resources(path)
+        cands.append((spec, path, res))
+        return res
+
+    for pd in (4, 2):
+        res = add(em.bw2(prefetch=pd))
+        if res is not None and res['occupancy'] < 4 and (res['occupancy'] < 2 or res['vgprs'] <= 224):
+            add(em.bw2(waves_per_simd=res['occupancy'] + 1, prefetch=pd))
+
+    def rank(c):
+        res = c[2]
+        if res is None:
+            return (1, 0, 0)
+        return (0 if res['scratch'] <= MAX_SPILL_BYTES else 1, -res['occupancy'], res['scratch'])
+
+    order = sorted(range(len(cands)), key=lambda i: (rank(cands[i]), i))
+    return [cands[i] for i in order]
 
 
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
-    """Emit + compile (or fetch from the cache) the kernels of a plan.  Needs no GPU.  With
-    `force` a cached code object is rebuilt, once per key recorded in `seen`.
-
-    The gradient kernel is register-hungry (a chunk of accumulators per lane) and hides memory
-    latency only through the waves resident on its SIMD.  After the plain build, builds that ask
-    the compiler for one more wave per SIMD are tried, and taken as long as they spill at most
-    `MAX_SPILL_BYTES` per lane; the compiler's own resource report decides, not a timing."""
-    def build(specs):
-        jobs = []
-        for s in specs:
-            key = runtime.source_key(s.name, s.source)
-            again = force and (seen is None or key not in seen)
-            if seen is not None:
-                seen.add(key)
-            jobs.append((s, again))
-        # independent compiler processes: wait for them side by side (the runtime call releases the GIL)
-        with ThreadPoolExecutor(max_workers=max(1, len(jobs))) as pool:
-            paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
-        return [(s, path) for (s, _), path in zip(jobs, paths)]
-
-    built = build(kernel_specs(plan))
-    if built[-1][0].name == 'frnn_bw2':
-        res = runtime.kernel_resources(built[-1][1])
-        em = Emitter(plan)
-        while res is not None and res['occupancy'] < 4 and res['vgprs'] <= 224:
-            cand = build([em.bw2(waves_per_simd=res['occupancy'] + 1)])[0]
-            cres = runtime.kernel_resources(cand[1])
-            if cres is None or cres['occupancy'] <= res['occupancy'] or cres['scratch'] > MAX_SPILL_BYTES:
-                break
-            built[-1], res = cand, cres
+    """Emit + compile (or fetch from the cache) the kernels of a plan, every candidate build of
+    the gradient kernel included; returns the forward kernel, the reverse scan and the
+    first-ranked gradient kernel.  Needs no GPU.  With `force` a cached code object is rebuilt,
+    once per key recorded in `seen`."""
+    em = Emitter(plan)
+    built = _compile([em.fw(), em.bw1()], force, seen)
+    if needs_gradient_kernel(plan.part):
+        spec, path, _ = gradient_kernel_builds(plan, force, seen)[0]
+        built.append((spec, path))
     return built
 
 
 class CompiledPlan:
+    _tune_pending = False
+
     def __init__(self, plan, state_meta=None):
         self.plan = plan
         # (shape, stride, dtype) of the initial states: gradients w.r.t. them are laid out alike
         self.state_meta = state_meta
         # when set to a list, every launch appends (kernel name, start event, end event)
         self.profile_events = None
-        built = compile_plan(plan)
+        em = Emitter(plan)
+        built = _compile([em.fw(), em.bw1()], False, None)
         self.kernels = {}
         self.modules = []
-        for spec, path in built:
+
+        def load(spec, path):
             try:
                 mod = runtime.Module(path)
                 kern = mod.kernel(spec.name)
@@ -89,7 +125,18 @@ class CompiledPlan:
                 mod = runtime.Module(path)
                 kern = mod.kernel(spec.name)
             self.modules.append(mod)
-            self.kernels[spec.name] = (spec, kern)
+            return kern
+
+        for spec, path in built:
+            self.kernels[spec.name] = (spec, load(spec, path))
+        # gradient kernel: every candidate build is loaded; the first backward call times them
+        self.bw2_builds = []
+        self.bw2_times = None
+        if needs_gradient_kernel(plan.part):
+            for spec, path, res in gradient_kernel_builds(plan):
+                self.bw2_builds.append((spec, load(spec, path), res))
+            self.kernels['frnn_bw2'] = self.bw2_builds[0][:2]
+        self._tune_pending = len(self.bw2_builds) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0'
         # per kernel: grid (fixed by the plan's sizes) and one packer for the whole argument block
         env = dict(B=plan.B, T=plan.T, H=plan.H, M=plan.M, nch=plan.nchunks)
         self._grid = {k: tuple(int(eval(g, {}, env)) for g in s.grid) for k, (s, _) in self.kernels.items()}
@@ -122,6 +169,28 @@ class CompiledPlan:
                 self.profile_events.append((kname, e0, e1))
             else:
                 kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
+
+    def _tune_gradient_kernel(self, tensors, accumulators):
+        """Times every candidate build of the gradient kernel once on the tensors of this call
+        (after one untimed run each) and keeps the fastest.  The kernel only stores and
+        accumulates; what it accumulated into is cleared again afterwards.  Synchronises."""
+        self._tune_pending = False
+        saved = [a.clone() for a in accumulators]       # the reverse scan has already added its share
+        times = []
+        for spec, kern, res in self.bw2_builds:
+            self.kernels['frnn_bw2'] = (spec, kern)
+            self._launch('frnn_bw2', tensors)
+            e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
+            e0.record()
+            self._launch('frnn_bw2', tensors)
+            e1.record()
+            e1.synchronize()
+            times.append(e0.elapsed_time(e1))
+        best = min(range(len(times)), key=times.__getitem__)
+        self.kernels['frnn_bw2'] = self.bw2_builds[best][:2]
+        self.bw2_times = times
+        for a, s_ in zip(accumulators, saved):
+            a.copy_(s_)
 
     # ------------------------------------------------------------------ forward
     def forward(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
@@ -177,6 +246,8 @@ class CompiledPlan:
             tensors[f'dout{k}'] = doutput[k]
         self._launch('frnn_bw1', tensors)
         if 'frnn_bw2' in self.kernels:
+            if self._tune_pending and not th.cuda.is_current_stream_capturing():
+                self._tune_gradient_kernel(tensors, [dins[i] for i in atomic])
             self._launch('frnn_bw2', tensors)
         for i in atomic:
             x = inputs[i]

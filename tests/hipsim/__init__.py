@@ -57,7 +57,8 @@ class SimPlan(CompiledPlan):
         self.state_meta = state_meta
         self.against_end = against_end
         self.kernels = {}
-        for spec in kernel_specs(plan):
+        # HIPSIM_PREFETCH selects the gradient kernel's variant with that many checkpoint rows in flight
+        for spec in kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4'))):
             lib = ctypes.CDLL(_compile_host(spec))
             lib.sim_alloc.restype = ctypes.c_void_p
             lib.sim_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]

@@ -70,7 +70,8 @@ TILED = [
 
 @pytest.mark.parametrize('case,dims,dtype,end,tile', TILED)
 def test_tile_overrides(case, dims, dtype, end, tile):
-    env = dict(os.environ, FLEX_RNN_TILE=tile)
+    # (these runs also take the gradient kernel's two-rows-in-flight variant)
+    env = dict(os.environ, FLEX_RNN_TILE=tile, HIPSIM_PREFETCH='2')
     r = subprocess.run([sys.executable, RUNNER, case, dims, dtype, str(end)], capture_output=True, text=True, timeout=900, env=env)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
     assert tile.split(',')[0] in r.stdout.replace(' ', '')
