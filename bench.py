@@ -90,6 +90,15 @@ def main():
             f(*xs, *ss)
         th.cuda.synchronize()
         fwd_ms = (time.perf_counter() - t1) * 1e3 / args.steps
+        # inference: the forward kernel that saves nothing for a backward pass
+        for _ in range(2):
+            f.infer(*xs, *ss)
+        th.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(args.steps):
+            f.infer(*xs, *ss)
+        th.cuda.synchronize()
+        inf_ms = (time.perf_counter() - t1) * 1e3 / args.steps
     ms_per_step = wall * 1e3 / args.steps
     tokens = B * T
     value = tokens / (wall / args.steps)
@@ -146,6 +155,7 @@ def main():
         'forward_only': {'ms_per_step': round(fwd_ms, 4), 'tokens_per_s': round(tokens / (fwd_ms * 1e-3), 1),
                          'achieved_TFLOPs': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12, 3),
                          'frac': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4)},
+        'inference': {'ms_per_step': round(inf_ms, 4), 'tokens_per_s': round(tokens / (inf_ms * 1e-3), 1)},
     }
     print(json.dumps(out))
 

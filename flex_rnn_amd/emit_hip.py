@@ -477,7 +477,9 @@ class Emitter:
         return f'(((i64)(b * H + h) * nch + ({chunk})) * M + (row0 + r)) * {N} + COL(c)'
 
     # ------------------------------------------------------------------ fw
-    def fw(self) -> KernelSpec:
+    def fw(self, save: bool = True) -> KernelSpec:
+        """Forward recurrence.  With `save=False` (inference: no backward pass will follow) the state
+        checkpoints and the per-step row sums are not written; the kernel is then named `frnn_fwi`."""
         p, plan, t = self.p, self.plan, self.tile
         L, C, G, R, W, DT, TS = t.L, t.C, t.G, t.R, t.W, t.DT, t.TS
         N = plan.N
@@ -485,6 +487,10 @@ class Emitter:
         A = _Args()
         g = p.fw
         nin, nst, nout, naux = p.ninputs, p.nstates, p.noutputs, len(p.aux)
+        kname = 'frnn_fw' if save else 'frnn_fwi'
+        if not save:
+            g = g.extract('fw', g.outputs[:nout + nst], cut=())
+            naux = 0
         out_exts = [(True, False)] * nout + [(True, True)] * nst + [(True, False)] * naux
         # a state of a problem with M == 1 or N == 1 has a smaller extent; follow the joint graph
         st_ext = [self.jext[s] for s in p.st_names]
@@ -524,7 +530,7 @@ class Emitter:
         body.append(f'  for (int t0 = 0; t0 < T; t0 += {TS}) {{\n')
         # checkpoint
         body.append(f'    if (t0 % {DT} == 0) {{\n')
-        for k in range(nst):
+        for k in range(nst if save else 0):
             rr, cc = _dims(st_ext[k], R, C)
             body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
@@ -589,10 +595,10 @@ class Emitter:
             body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) stf<{dt}>({A.p(nm)}, '
                         f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, S{k}[r][c]); }}\n')
-        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_fw(Args A) {{\n'
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) {kname}(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
         source = PRELUDE + A.struct() + fn_src + '\n' + kernel
-        return KernelSpec('frnn_fw', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
+        return KernelSpec(kname, source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
 
     # ------------------------------------------------------------------ bw1
     def bw1(self) -> KernelSpec:

@@ -77,6 +77,22 @@ class jit:
         assert key in self._bw_index, 'backward called with tensors no forward call has produced'
         return self._bw_index[key]
 
+    def infer(self, *args):
+        """Outputs and final states without the ability to differentiate: the forward kernel then
+        writes neither state checkpoints nor the per-step row sums the backward pass would need
+        (an addition to the reference's interface, for inference and decoding loops).  Same
+        arguments and results as a call; not recorded by autograd."""
+        inputs, state = split_list(args, [self.ninputs, self.nstates])
+        with th.no_grad():
+            if self.is_dynamic:
+                fwd = self._entry(inputs, state, dry=False)['forward']
+            else:
+                if self.forward_func is None:
+                    self.forward_func, self.backward_func, self.fw_meta, self.bw_meta = \
+                        build_twopass(self.step, inputs, state)
+                fwd = self.forward_func
+            return fwd.forward_only(inputs, state)
+
     # ------------------------------------------------------------------ oracle
     def naive(self, *args, dtype=th.float32):
         """Pure-PyTorch per-timestep loop with the compiled path's calling convention

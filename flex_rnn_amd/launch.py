@@ -92,7 +92,7 @@ def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec,
     first-ranked gradient kernel.  Needs no GPU.  With `force` a cached code object is rebuilt,
     once per key recorded in `seen`."""
     em = Emitter(plan)
-    built = _compile([em.fw(), em.bw1()], force, seen)
+    built = _compile([em.fw(), em.bw1(), em.fw(save=False)], force, seen)[:2]
     if needs_gradient_kernel(plan.part):
         spec, path, _ = gradient_kernel_builds(plan, force, seen)[0]
         built.append((spec, path))
@@ -127,6 +127,7 @@ class CompiledPlan:
             self.modules.append(mod)
             return kern
 
+        self._load = load
         for spec, path in built:
             self.kernels[spec.name] = (spec, load(spec, path))
         # gradient kernel: every candidate build is loaded; the first backward call times them
@@ -138,9 +139,20 @@ class CompiledPlan:
             self.kernels['frnn_bw2'] = self.bw2_builds[0][:2]
         self._tune_pending = len(self.bw2_builds) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0'
         # per kernel: grid (fixed by the plan's sizes) and one packer for the whole argument block
-        env = dict(B=plan.B, T=plan.T, H=plan.H, M=plan.M, nch=plan.nchunks)
-        self._grid = {k: tuple(int(eval(g, {}, env)) for g in s.grid) for k, (s, _) in self.kernels.items()}
-        self._packer = {k: struct.Struct('<' + 'q5q' * max(len(s.tensors), 1) + '5q') for k, (s, _) in self.kernels.items()}
+        self._grid, self._packer = {}, {}
+        for k, (s, _) in self.kernels.items():
+            self._register(k, s)
+
+    def _register(self, name, spec):
+        pl = self.plan
+        env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
+        self._grid[name] = tuple(int(eval(g, {}, env)) for g in spec.grid)
+        self._packer[name] = struct.Struct('<' + 'q5q' * max(len(spec.tensors), 1) + '5q')
+
+    def _add_kernel(self, spec):
+        path = _compile([spec], False, None)[0][1]
+        self.kernels[spec.name] = (spec, self._load(spec, path))
+        self._register(spec.name, spec)
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
@@ -212,6 +224,26 @@ class CompiledPlan:
             tensors[f'out{k}'] = outs[k]
         self._launch('frnn_fw', tensors)
         return (*outs, *stT, *sck, aux)
+
+    def forward_only(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
+        """Outputs and final states only (inference): a forward kernel that writes no checkpoints and
+        no saved row sums, built on first use."""
+        if 'frnn_fwi' not in self.kernels:
+            self._add_kernel(Emitter(self.plan).fw(save=False))
+        pl, p = self.plan, self.plan.part
+        dev = inputs[0].device
+        outs = tuple(th.empty(pl.B, pl.T, pl.H, pl.M, dtype=dt, device=dev) for dt in pl.out_dtypes)
+        stT = tuple(th.empty_like(s) for s in state0)
+        tensors = {}
+        for i, x in enumerate(inputs):
+            tensors[f'in{i}'] = x
+        for k in range(p.nstates):
+            tensors[f'st{k}'] = state0[k]
+            tensors[f'stT{k}'] = stT[k]
+        for k in range(p.noutputs):
+            tensors[f'out{k}'] = outs[k]
+        self._launch('frnn_fwi', tensors)
+        return (*outs, *stT)
 
     # ------------------------------------------------------------------ backward
     def backward(self, doutput, dstateT, inputs, state_store, aux):

@@ -324,5 +324,11 @@ def build_twopass(step: Callable, inputs, state, dryrun: bool = False, tile: Opt
         verify_meta(aux_, fw_out_meta[nout + 2 * nst:])
         return compiled.backward(doutput, dstateT_, tuple(inputs_), tuple(state_store_), aux_[0])
 
+    def forward_only(inputs_, state0):
+        verify_meta(inputs_, in_meta, 'input Tensor metadata doesn\'t match compilation\n')
+        verify_meta(state0, st_meta, 'initial state Tensor metadata doesn\'t match compilation\n')
+        return compiled.forward_only(tuple(inputs_), tuple(state0))
+
     forward.compiled = backward.compiled = compiled
+    forward.forward_only = forward_only
     return forward, backward, forward_meta, backward_meta

@@ -59,13 +59,16 @@ class SimPlan(CompiledPlan):
         self.kernels = {}
         # HIPSIM_PREFETCH selects the gradient kernel's variant with that many checkpoint rows in flight
         for spec in kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4'))):
-            lib = ctypes.CDLL(_compile_host(spec))
-            lib.sim_alloc.restype = ctypes.c_void_p
-            lib.sim_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]
-            lib.sim_free.argtypes = [ctypes.c_void_p]
-            fn = getattr(lib, f'sim_launch_{spec.name}')
-            fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-            self.kernels[spec.name] = (spec, lib, fn)
+            self._add_kernel(spec)
+
+    def _add_kernel(self, spec):
+        lib = ctypes.CDLL(_compile_host(spec))
+        lib.sim_alloc.restype = ctypes.c_void_p
+        lib.sim_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]
+        lib.sim_free.argtypes = [ctypes.c_void_p]
+        fn = getattr(lib, f'sim_launch_{spec.name}')
+        fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        self.kernels[spec.name] = (spec, lib, fn)
 
     def _launch(self, kname, tensors):
         spec, lib, fn = self.kernels[kname]

@@ -46,6 +46,10 @@ def main():
     sp = SimPlan(plan, state_meta=fm[nout:nout + nst], against_end=bool(end))
     res = sp.forward(tuple(xs), tuple(ss))
     outs, stT, sck, aux = res[:nout], res[nout:nout + nst], res[nout + nst:nout + 2 * nst], res[-1]
+    # the inference kernel (no checkpoints, no saved sums) must give the same outputs and final states
+    lean = sp.forward_only(tuple(xs), tuple(ss))
+    for a, b in zip(lean, list(outs) + list(stT)):
+        assert th.equal(a, b) or recurrence.rel_err(a, b) < 1e-6, 'forward_only differs from forward'
     g = th.Generator().manual_seed(11)
     dy = [th.randn(o.shape, generator=g) for o in outs]
     dS = [th.randn(s.shape, generator=g) for s in ss]

@@ -115,6 +115,16 @@ def test_dynamic_mode_plans_one_entry_per_signature():
     assert tuple(y.shape) == (2, 16, 2, 8)
 
 
+def test_infer_is_part_of_the_surface_and_has_no_cpu_fallback(runtime_lib):
+    if th.cuda.is_available():
+        pytest.skip('a GPU is present')
+    f = flex_rnn_amd.jit(ops.delta_rule)
+    step, xs, ss = cases.make_inputs('delta_rule', 2, 16, 2, 8, 8, dtype=th.float32)
+    with pytest.raises(Exception) as e:
+        f.infer(*xs, *ss)
+    assert 'GPU' in str(e.value) or 'HIP' in str(e.value) or 'hip' in str(e.value)
+
+
 def test_compiled_path_has_no_cpu_fallback(runtime_lib):
     if th.cuda.is_available():
         pytest.skip('a GPU is present')

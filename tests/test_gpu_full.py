@@ -141,6 +141,20 @@ def test_dynamic_mode_accepts_other_shapes():
     assert len(f._entries) == 3
 
 
+@pytest.mark.parametrize('name', ['rwkv7', 'mamba1', 'mamba2'])
+def test_infer_matches_call(name):
+    """`jit.infer` (no checkpoints, no saved sums) returns what a normal call returns."""
+    print(f'case infer {name}', flush=True)
+    B, T, H, M, N = configs.DEFAULT_DIMS[name]
+    wl = configs.make(name, dims=(2, 77, 2, M, N))
+    f = flex_rnn_amd.jit(wl.step)
+    xs, ss = _gpu(wl.inputs), _gpu(wl.states)
+    a = f.infer(*xs, *ss)
+    b = f(*xs, *ss)
+    assert len(a) == len(b) and all(th.equal(x, y) for x, y in zip(a, b))
+    assert not any(t.requires_grad for t in a)
+
+
 def test_torch_compile_no_graph_break():
     print('case torch.compile', flush=True)
     step, xs, ss = cases.make_inputs('delta_rule', 2, 32, 2, 16, 16, dtype=th.float32)
