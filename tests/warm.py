@@ -72,6 +72,10 @@ def warm(force=False, seen=None):
         B, T, H, M, N = configs.DEFAULT_DIMS[name]
         n += len(compile_plan(prebuild.plan_for(name, (B, 128, H, M, N)), force=force, seen=seen))
     n += len(compile_plan(prebuild.plan_for('rwkv7', (8, 512, 32, 128, 128)), force=force, seen=seen))
+    n += len(compile_plan(prebuild.plan_for('mamba2', (2, 64, 4, 64, 128)), force=force, seen=seen))
+    for name in ('rwkv7', 'mamba1', 'mamba2'):
+        B, T, H, M, N = configs.DEFAULT_DIMS[name]
+        n += len(compile_plan(prebuild.plan_for(name, (2, 77, 2, M, N)), force=force, seen=seen))
     for name, dims in [('rwkv7', (2, 77, 2, 128, 128)), ('mamba1', (2, 45, 4, 128, 16)),
                        ('gated_delta_rule', (2, 1, 2, 128, 128)), ('mamba2', (2, 19, 4, 64, 128))]:
         n += len(compile_plan(prebuild.plan_for(name, dims, th.float32), force=force, seen=seen))
