@@ -47,7 +47,7 @@ def main():
 
     import torch as th
     import flex_rnn_amd
-    from flex_rnn_amd import configs
+    from flex_rnn_amd import configs, launch
 
     assert th.cuda.is_available(), 'bench.py needs a GPU'
     dev = th.device('cuda:0')
@@ -148,6 +148,9 @@ def main():
         'roofline': roofline, 'cpu_baseline': cpu,
         'gpu_kernel_ms_per_step': round(gpu_ms, 4),
         # candidate builds of the gradient kernel as timed on the first backward call (the fastest runs)
+        'row_kernel_builds': {k: {'rows_per_lane, waves': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
+                                  'ms': compiled.build_times.get(k) and [round(v, 4) for v in compiled.build_times[k]]}
+                              for k in ('frnn_fw', 'frnn_bw1')},
         'gradient_kernel_builds': [
             {'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
              'ms': compiled.bw2_times and round(compiled.bw2_times[i], 4)}

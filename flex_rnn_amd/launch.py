@@ -10,6 +10,7 @@ fp32 scratch + cast-back for gradients of inputs broadcast over batch / time / h
 """
 from __future__ import annotations
 
+import dataclasses
 import os
 import struct
 from concurrent.futures import ThreadPoolExecutor
@@ -86,13 +87,39 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
     return [cands[i] for i in order]
 
 
+def row_kernel_tiles(plan, reverse: bool):
+    """(R, W) candidates for the forward kernel (or the reverse scan): the heuristic's choice first,
+    then half the rows per lane (more, lighter waves) with the same and with twice the waves per
+    workgroup.  Which is fastest depends on how many (batch, head) pairs there are, on the LDS
+    traffic of the staged operands and on register use; the first call times them."""
+    t = plan.tile
+    R, W = ((t.R1 or t.R), (t.W1 or t.W)) if reverse else (t.R, t.W)
+    G = t.G
+    out = [(R, W)]
+    fixed_r = reverse and plan.part.dstep_needs_state          # one row per lane there (register budget)
+    for r, w in ((R // 2, W), (R // 2, 2 * W)) if (R > 1 and not fixed_r) else ((R, 2 * W),):
+        if r >= 1 and w <= 8 and w * G * r <= max(plan.M, G * r) and (r, w) not in out:
+            out.append((r, w))
+    return out
+
+
+def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None):
+    """[(spec, path)] for `row_kernel_tiles`, compiled side by side."""
+    specs = []
+    for r, w in row_kernel_tiles(plan, reverse):
+        tile = dataclasses.replace(plan.tile, R1=r, W1=w) if reverse else dataclasses.replace(plan.tile, R=r, W=w)
+        em = Emitter(dataclasses.replace(plan, tile=tile))
+        specs.append(em.bw1() if reverse else em.fw())
+    return _compile(specs, force, seen)
+
+
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
     """Emit + compile (or fetch from the cache) the kernels of a plan, every candidate build of
     the gradient kernel included; returns the forward kernel, the reverse scan and the
     first-ranked gradient kernel.  Needs no GPU.  With `force` a cached code object is rebuilt,
     once per key recorded in `seen`."""
-    em = Emitter(plan)
-    built = _compile([em.fw(), em.bw1(), em.fw(save=False)], force, seen)[:2]
+    built = [row_kernel_builds(plan, False, force, seen)[0], row_kernel_builds(plan, True, force, seen)[0]]
+    _compile([Emitter(plan).fw(save=False)], force, seen)
     if needs_gradient_kernel(plan.part):
         spec, path, _ = gradient_kernel_builds(plan, force, seen)[0]
         built.append((spec, path))
@@ -100,7 +127,7 @@ def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec,
 
 
 class CompiledPlan:
-    _tune_pending = False
+    _tune_pending = frozenset()
 
     def __init__(self, plan, state_meta=None):
         self.plan = plan
@@ -108,8 +135,6 @@ class CompiledPlan:
         self.state_meta = state_meta
         # when set to a list, every launch appends (kernel name, start event, end event)
         self.profile_events = None
-        em = Emitter(plan)
-        built = _compile([em.fw(), em.bw1()], False, None)
         self.kernels = {}
         self.modules = []
 
@@ -128,20 +153,32 @@ class CompiledPlan:
             return kern
 
         self._load = load
-        for spec, path in built:
-            self.kernels[spec.name] = (spec, load(spec, path))
-        # gradient kernel: every candidate build is loaded; the first backward call times them
-        self.bw2_builds = []
-        self.bw2_times = None
+        # Every kernel comes in a few candidate builds (tiles of the row kernels; prefetch depth and
+        # occupancy request of the gradient kernel), first-ranked first.  All are loaded; the first
+        # call that runs a kernel times its candidates on that call's tensors and keeps the fastest.
+        self.builds = {'frnn_fw': [(s_, load(s_, p_), None) for s_, p_ in row_kernel_builds(plan, False)],
+                       'frnn_bw1': [(s_, load(s_, p_), None) for s_, p_ in row_kernel_builds(plan, True)]}
         if needs_gradient_kernel(plan.part):
-            for spec, path, res in gradient_kernel_builds(plan):
-                self.bw2_builds.append((spec, load(spec, path), res))
-            self.kernels['frnn_bw2'] = self.bw2_builds[0][:2]
-        self._tune_pending = len(self.bw2_builds) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0'
-        # per kernel: grid (fixed by the plan's sizes) and one packer for the whole argument block
+            self.builds['frnn_bw2'] = [(s_, load(s_, p_), r_) for s_, p_, r_ in gradient_kernel_builds(plan)]
+        self.build_times = {}
+        tune = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
+        self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1}
         self._grid, self._packer = {}, {}
-        for k, (s, _) in self.kernels.items():
-            self._register(k, s)
+        for k, v in self.builds.items():
+            self._select(k, 0)
+
+    @property
+    def bw2_builds(self):
+        return self.builds.get('frnn_bw2', [])
+
+    @property
+    def bw2_times(self):
+        return self.build_times.get('frnn_bw2')
+
+    def _select(self, name, index):
+        spec, kern, _ = self.builds[name][index]
+        self.kernels[name] = (spec, kern)
+        self._register(name, spec)
 
     def _register(self, name, spec):
         pl = self.plan
@@ -182,25 +219,30 @@ class CompiledPlan:
             else:
                 kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
 
-    def _tune_gradient_kernel(self, tensors, accumulators):
-        """Times every candidate build of the gradient kernel once on the tensors of this call
-        (after one untimed run each) and keeps the fastest.  The kernel only stores and
-        accumulates; what it accumulated into is cleared again afterwards.  Synchronises."""
-        self._tune_pending = False
-        saved = [a.clone() for a in accumulators]       # the reverse scan has already added its share
+    def _tune(self, name, tensors, accumulators=()):
+        """Times every candidate build of kernel `name` on the tensors of this call (one untimed
+        run, then the faster of two timed ones) and keeps the fastest.  The kernels only store and
+        accumulate; `accumulators` (what they add into) are put back afterwards.  Synchronises,
+        once per kernel and plan; skipped while the stream is being captured."""
+        if name not in self._tune_pending or th.cuda.is_current_stream_capturing():
+            return
+        self._tune_pending.discard(name)
+        saved = [a.clone() for a in accumulators]
         times = []
-        for spec, kern, res in self.bw2_builds:
-            self.kernels['frnn_bw2'] = (spec, kern)
-            self._launch('frnn_bw2', tensors)
-            e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
-            e0.record()
-            self._launch('frnn_bw2', tensors)
-            e1.record()
-            e1.synchronize()
-            times.append(e0.elapsed_time(e1))
-        best = min(range(len(times)), key=times.__getitem__)
-        self.kernels['frnn_bw2'] = self.bw2_builds[best][:2]
-        self.bw2_times = times
+        for i in range(len(self.builds[name])):
+            self._select(name, i)
+            self._launch(name, tensors)
+            best = float('inf')
+            for _ in range(2):
+                e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
+                e0.record()
+                self._launch(name, tensors)
+                e1.record()
+                e1.synchronize()
+                best = min(best, e0.elapsed_time(e1))
+            times.append(best)
+        self._select(name, min(range(len(times)), key=times.__getitem__))
+        self.build_times[name] = times
         for a, s_ in zip(accumulators, saved):
             a.copy_(s_)
 
@@ -222,6 +264,7 @@ class CompiledPlan:
             tensors[f'sck{k}'] = sck[k]
         for k in range(p.noutputs):
             tensors[f'out{k}'] = outs[k]
+        self._tune('frnn_fw', tensors)
         self._launch('frnn_fw', tensors)
         return (*outs, *stT, *sck, aux)
 
@@ -229,7 +272,7 @@ class CompiledPlan:
         """Outputs and final states only (inference): a forward kernel that writes no checkpoints and
         no saved row sums, built on first use."""
         if 'frnn_fwi' not in self.kernels:
-            self._add_kernel(Emitter(self.plan).fw(save=False))
+            self._add_kernel(Emitter(self.plan).fw(save=False))       # (the heuristic's tile)
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
         outs = tuple(th.empty(pl.B, pl.T, pl.H, pl.M, dtype=dt, device=dev) for dt in pl.out_dtypes)
@@ -276,10 +319,11 @@ class CompiledPlan:
                 tensors[f'dck{k}'] = dck[k]
         for k in range(p.noutputs):
             tensors[f'dout{k}'] = doutput[k]
+        acc = [dins[i] for i in atomic]             # zero so far; each kernel adds its own inputs' gradients
+        self._tune('frnn_bw1', tensors, acc)
         self._launch('frnn_bw1', tensors)
         if 'frnn_bw2' in self.kernels:
-            if self._tune_pending and not th.cuda.is_current_stream_capturing():
-                self._tune_gradient_kernel(tensors, [dins[i] for i in atomic])
+            self._tune('frnn_bw2', tensors, acc)
             self._launch('frnn_bw2', tensors)
         for i in atomic:
             x = inputs[i]

@@ -65,6 +65,10 @@ TILED = [
     ('cfg:mamba2', '2,21,2,7,128', 'bf16', 1, 'MS=3'),
     ('cfg:mamba2', '2,16,4,16,128', 'f32', 0, 'HB=2,MS=1'),
     ('cfg:mamba2', '2,16,4,16,128', 'f32', 1, 'HB=4,MS=2'),
+    # row-kernel tiles that the first-call timing may pick instead of the heuristic's
+    ('cfg:rwkv7', '1,16,2,128,128', 'f32', 0, 'R=2,W=8,R1=2,W1=4'),
+    ('cfg:mamba2', '2,16,2,64,128', 'f32', 1, 'R=1,W=8,R1=1,W1=8'),
+    ('cfg:mamba1', '2,16,2,128,16', 'f32', 0, 'R=1,W=8,R1=1,W1=8'),
 ]
 
 
