@@ -103,13 +103,14 @@ def row_kernel_tiles(plan, reverse: bool):
     return out
 
 
-def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None):
-    """[(spec, path)] for `row_kernel_tiles`, compiled side by side."""
+def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save: bool = True):
+    """[(spec, path)] for `row_kernel_tiles`, compiled side by side (`save=False`: the inference
+    variant of the forward kernel)."""
     specs = []
     for r, w in row_kernel_tiles(plan, reverse):
         tile = dataclasses.replace(plan.tile, R1=r, W1=w) if reverse else dataclasses.replace(plan.tile, R=r, W=w)
         em = Emitter(dataclasses.replace(plan, tile=tile))
-        specs.append(em.bw1() if reverse else em.fw())
+        specs.append(em.bw1() if reverse else em.fw(save=save))
     return _compile(specs, force, seen)
 
 
@@ -119,7 +120,7 @@ def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec,
     first-ranked gradient kernel.  Needs no GPU.  With `force` a cached code object is rebuilt,
     once per key recorded in `seen`."""
     built = [row_kernel_builds(plan, False, force, seen)[0], row_kernel_builds(plan, True, force, seen)[0]]
-    _compile([Emitter(plan).fw(save=False)], force, seen)
+    row_kernel_builds(plan, False, force, seen, save=False)
     if needs_gradient_kernel(plan.part):
         spec, path, _ = gradient_kernel_builds(plan, force, seen)[0]
         built.append((spec, path))
@@ -186,10 +187,11 @@ class CompiledPlan:
         self._grid[name] = tuple(int(eval(g, {}, env)) for g in spec.grid)
         self._packer[name] = struct.Struct('<' + 'q5q' * max(len(spec.tensors), 1) + '5q')
 
-    def _add_kernel(self, spec):
-        path = _compile([spec], False, None)[0][1]
-        self.kernels[spec.name] = (spec, self._load(spec, path))
-        self._register(spec.name, spec)
+    def _add_builds(self, name, built):
+        self.builds[name] = [(s_, self._load(s_, p_), r_) for s_, p_, r_ in built]
+        if len(built) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0':
+            self._tune_pending.add(name)
+        self._select(name, 0)
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
@@ -272,7 +274,7 @@ class CompiledPlan:
         """Outputs and final states only (inference): a forward kernel that writes no checkpoints and
         no saved row sums, built on first use."""
         if 'frnn_fwi' not in self.kernels:
-            self._add_kernel(Emitter(self.plan).fw(save=False))       # (the heuristic's tile)
+            self._add_builds('frnn_fwi', [(s_, p_, None) for s_, p_ in row_kernel_builds(self.plan, False, save=False)])
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
         outs = tuple(th.empty(pl.B, pl.T, pl.H, pl.M, dtype=dt, device=dev) for dt in pl.out_dtypes)
@@ -285,6 +287,7 @@ class CompiledPlan:
             tensors[f'stT{k}'] = stT[k]
         for k in range(p.noutputs):
             tensors[f'out{k}'] = outs[k]
+        self._tune('frnn_fwi', tensors)
         self._launch('frnn_fwi', tensors)
         return (*outs, *stT)
 

@@ -61,6 +61,12 @@ class SimPlan(CompiledPlan):
         for spec in kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4'))):
             self._add_kernel(spec)
 
+    def _add_builds(self, name, built):
+        self._add_kernel(built[0][0])
+
+    def _tune(self, name, tensors, accumulators=()):
+        pass
+
     def _add_kernel(self, spec):
         lib = ctypes.CDLL(_compile_host(spec))
         lib.sim_alloc.restype = ctypes.c_void_p
