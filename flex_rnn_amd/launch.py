@@ -63,19 +63,22 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
     em = Emitter(plan)
     cands, seen_src = [], set()
 
-    def add(spec):
-        if spec.source in seen_src:
-            return None
-        seen_src.add(spec.source)
-        path = _compile([spec], force, seen)[0][1]
-        res = runtime.kernel_resources(path)
-        cands.append((spec, path, res))
-        return res
+    def add(specs):
+        specs = [sp for sp in specs if sp.source not in seen_src and not seen_src.add(sp.source)]
+        out = []
+        for spec, path in _compile(specs, force, seen):
+            res = runtime.kernel_resources(path)
+            cands.append((spec, path, res))
+            out.append(res)
+        return out
 
-    for pd in (4, 2):
-        res = add(em.bw2(prefetch=pd))
+    depths = (4, 2)
+    plain = add([em.bw2(prefetch=pd) for pd in depths])
+    more = []
+    for pd, res in zip(depths, plain):          # (a duplicate source was dropped: zip stops short, which is fine)
         if res is not None and res['occupancy'] < 4 and (res['occupancy'] < 2 or res['vgprs'] <= 224):
-            add(em.bw2(waves_per_simd=res['occupancy'] + 1, prefetch=pd))
+            more.append(em.bw2(waves_per_simd=res['occupancy'] + 1, prefetch=pd))
+    add(more)
 
     def rank(c):
         res = c[2]
@@ -157,10 +160,13 @@ class CompiledPlan:
         # Every kernel comes in a few candidate builds (tiles of the row kernels; prefetch depth and
         # occupancy request of the gradient kernel), first-ranked first.  All are loaded; the first
         # call that runs a kernel times its candidates on that call's tensors and keeps the fastest.
-        self.builds = {'frnn_fw': [(s_, load(s_, p_), None) for s_, p_ in row_kernel_builds(plan, False)],
-                       'frnn_bw1': [(s_, load(s_, p_), None) for s_, p_ in row_kernel_builds(plan, True)]}
-        if needs_gradient_kernel(plan.part):
-            self.builds['frnn_bw2'] = [(s_, load(s_, p_), r_) for s_, p_, r_ in gradient_kernel_builds(plan)]
+        with ThreadPoolExecutor(max_workers=3) as pool:         # compiler runs; loading happens on this thread
+            jobs = {'frnn_fw': pool.submit(lambda: [(s_, p_, None) for s_, p_ in row_kernel_builds(plan, False)]),
+                    'frnn_bw1': pool.submit(lambda: [(s_, p_, None) for s_, p_ in row_kernel_builds(plan, True)])}
+            if needs_gradient_kernel(plan.part):
+                jobs['frnn_bw2'] = pool.submit(gradient_kernel_builds, plan)
+            built = {k: j.result() for k, j in jobs.items()}
+        self.builds = {k: [(s_, load(s_, p_), r_) for s_, p_, r_ in v] for k, v in built.items()}
         self.build_times = {}
         tune = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
         self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1}
