@@ -143,7 +143,8 @@ def _loops(rr, cc):
 
 
 def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple[bool, bool]],
-                  reduce_fn: str, invariant: Sequence[str] = ()) -> Tuple[str, List[str]]:
+                  reduce_fn: str, invariant: Sequence[str] = (), colmask: str = '',
+                  prolog: str = '') -> Tuple[str, List[str]]:
     """Device function evaluating `g` on register tiles.  Every value is a `float[RR][CC]`
     array with RR = R if it varies along rows else 1, CC likewise for columns.  Returns the
     source and the list of graph inputs that appear in the signature (the used ones).
@@ -151,7 +152,10 @@ def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple
     `invariant` names graph inputs that do not change from one timestep to the next.
     `exp(u * v)` with such a `v` is evaluated as `exp2(u * (v * log2 e))`: the hardware
     exponential is base 2, and the rescaled `v` is loop-invariant for the compiler to hoist,
-    which saves the multiply by log2 e on every step."""
+    which saves the multiply by log2 e on every step.
+
+    `colmask` (an expression in `c`, or empty) is true for real state columns; with a state width
+    that is not a power of two the padding columns are kept out of every sum by it."""
     ext = g.ext_table()
     nm = g.node_map()
     invariant = set(invariant)
@@ -159,6 +163,8 @@ def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple
     params = [_ref(i, g.input_ext[i], R, C, True) for i in used]
     params += [_ref(f'o{k}_', e, R, C, False) for k, e in enumerate(out_exts)]
     out = [f'__device__ __forceinline__ void {fname}(' + ', '.join(params) + ') {']
+    if prolog:
+        out.append('  ' + prolog)
     for n in g.nodes:
         rr, cc = _dims(n.ext, R, C)
         out.append(f'  float {n.name}[{rr}][{cc}];')
@@ -173,9 +179,10 @@ def emit_graph_fn(g: Graph, fname: str, R: int, C: int, out_exts: Sequence[Tuple
             assert sext[1]
             srr = R if sext[0] else 1
             s_at = f"{src}[{'r' if sext[0] else '0'}]"
+            term = (lambda c: f'(({colmask.replace("(c)", f"({c})")}) ? {s_at}[{c}] : 0.0f)') if colmask else (lambda c: f'{s_at}[{c}]')
             out.append(f'#pragma unroll\n  for (int r = 0; r < {srr}; r++) {{\n'
-                       f'    float s_ = {s_at}[0];\n'
-                       f'#pragma unroll\n    for (int c = 1; c < {C}; c++) s_ += {s_at}[c];\n'
+                       f'    float s_ = {term("0")};\n'
+                       f'#pragma unroll\n    for (int c = 1; c < {C}; c++) s_ += {term("c")};\n'
                        f'    {n.name}[r][0] = {reduce_fn}(s_);\n  }}')
         elif n.op == 'const':
             out.append(f'  {n.name}[0][0] = {_lit(n.args[0])};')
@@ -250,18 +257,24 @@ class _Stager:
         self.TS, self.NT, self.tail = TS, NT, tail
         self.items = []      # (lds name, row length, dtype code, pointer, index fn(t, x_), time stride)
         self.no_lds = set()  # items that only feed derived operands: prefetched, never written to LDS
+        self.width = {}      # LDS row width per item (>= its row length)
         self.derived = None  # (function name, [source item names], [derived lds names], row length)
 
-    def add(self, name, ln, dt, ptr, idx_fn, tstride, lds=True):
+    def add(self, name, ln, dt, ptr, idx_fn, tstride, lds=True, width=None):
+        """`width` > `ln`: the LDS rows are that wide and the surplus (padding columns of a state
+        width that is not a power of two) is zeroed once, by `zero_pads()`."""
         self.items.append((name, ln, dt, ptr, idx_fn, tstride))
+        self.width[name] = width or ln
         if not lds:
             self.no_lds.add(name)
 
-    def derive(self, fn_name, sources, outputs, ln):
+    def derive(self, fn_name, sources, outputs, ln, width=None):
         """Operands computed while staging: `fn_name(src..., out...)` is evaluated once per
         (timestep, position) from the converted prefetch registers of `sources` (items of row
         length `ln`) and its results are written to the LDS arrays `outputs`."""
         self.derived = (fn_name, list(sources), list(outputs), ln)
+        for o in outputs:
+            self.width[o] = width or ln
 
     def _iters(self, ln):
         return (self.TS * ln + self.NT - 1) // self.NT
@@ -273,11 +286,25 @@ class _Stager:
         out = ''
         for name, ln, dt, ptr, fn, ts in self.items:
             if name not in self.no_lds:
-                out += f'  __shared__ float {name}[{self.TS}][{ln}];\n'
+                out += f'  __shared__ float {name}[{self.TS}][{self.width[name]}];\n'
             out += f'  unsigned pf_{name}[{self._iters(ln)}];\n'
         if self.derived:
             for o in self.derived[2]:
-                out += f'  __shared__ float {o}[{self.TS}][{self.derived[3]}];\n'
+                out += f'  __shared__ float {o}[{self.TS}][{self.width[o]}];\n'
+        return out
+
+    def zero_pads(self) -> str:
+        """Clears the padding columns of every LDS array wider than its operand (nothing else ever
+        writes them); a barrier must follow before the arrays are read."""
+        out = ''
+        arrays = [(name, ln) for name, ln, *_ in self.items if name not in self.no_lds]
+        if self.derived:
+            arrays += [(o, self.derived[3]) for o in self.derived[2]]
+        for name, ln in arrays:
+            pad = self.width[name] - ln
+            if pad > 0:
+                out += (f'  for (int e_ = tid; e_ < {self.TS * pad}; e_ += {self.NT}) '
+                        f'{name}[e_ / {pad}][{ln} + e_ % {pad}] = 0.0f;\n')
         return out
 
     def bases(self) -> str:
@@ -355,6 +382,10 @@ class Emitter:
         # (when T == 1 every non-matrix input counts as time-dependent, with a single step)
         self.tdep = [(plan.T == 1 or not b[1]) and c != 'mat' for b, c in zip(plan.in_bcast, self.cls)]
         self.atomic = set(plan.atomic)
+        # state width: N as given, NP as laid out (next power of two); `pad` when they differ
+        self.N, self.NP = plan.N, plan.NP
+        self.pad = plan.NP != plan.N
+        self.colmask = f'COL(c) < {plan.N}' if self.pad else ''
         self.invariant = {nm for nm, td in zip(p.in_names, self.tdep) if not td}
         self.jext = p.joint.ext_table()
         # the last chunk is partial when T is not a multiple of the chunk sizes; the guards that
@@ -414,9 +445,10 @@ class Emitter:
                 ext = self.in_ext(i)
                 assert ext == (False, True)
                 dt = DT_CODE[self.plan.in_dtypes[i]]
-                stg.add(f's_in{i}', self.plan.N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x),
-                        A.s(f'in{i}', 1), lds=p.in_names[i] in direct_used)
-        stg.derive(fn_name, [f's_in{p.in_names.index(v)}' for v in used], [f's_d{q}' for q in range(len(front))], self.plan.N)
+                stg.add(f's_in{i}', self.N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x),
+                        A.s(f'in{i}', 1), lds=p.in_names[i] in direct_used, width=self.NP)
+        stg.derive(fn_name, [f's_in{p.in_names.index(v)}' for v in used], [f's_d{q}' for q in range(len(front))],
+                   self.N, width=self.NP)
         return src
 
     def _row_kernel_common(self, R: int, W: int):
@@ -432,18 +464,28 @@ class Emitter:
   const int row0 = mt * {MT} + rloc;
   const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T; (void)H; (void)nch;
-#define COL(c) {_col_expr(C, L)}
-#define ROWC(r) (min(row0 + (r), M - 1))
 ''')
         return src, MT
 
+    def _row_macros(self) -> str:
+        """File-scope macros of the row kernels: column of (lane-in-group `l`, element c), the same
+        clamped to the real width, and the clamped row."""
+        t = self.tile
+        return (f'#define COL(c) {_col_expr(t.C, t.L)}\n'
+                f'#define COLC(c) {f"(min(COL(c), {self.N - 1}))" if self.pad else "COL(c)"}\n'
+                '#define ROWC(r) (min(row0 + (r), M - 1))\n')
+
+    def _lane_prolog(self) -> str:
+        """What a device function needs to evaluate COL(c) on its own (only emitted with padding)."""
+        return f'const int l = (threadIdx.x & 63) % {self.tile.L};' if self.pad else ''
+
     def _stage_input(self, st: '_Stager', A: _Args, i: int, MT: int):
         ext = self.in_ext(i)
-        N = self.plan.N
+        N = self.N
         dt = DT_CODE[self.plan.in_dtypes[i]]
         ts = A.s(f'in{i}', 1)
         if ext == (False, True):
-            st.add(f's_in{i}', N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x), ts)
+            st.add(f's_in{i}', N, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt, n=x), ts, width=self.NP)
         elif ext == (True, False):
             st.add(f's_in{i}', MT, dt, A.p(f'in{i}'),
                    lambda tt, x, i=i: self._in_index(A, i, t=tt, m=f'min(mt * {MT} + {x}, M - 1)'), ts)
@@ -468,13 +510,21 @@ class Emitter:
         ext = self.in_ext(i)
         rr, cc = _dims(ext, R, C)
         dt = DT_CODE[self.plan.in_dtypes[i]]
-        idx = self._in_index(A, i, t='0', m='ROWC(r)' if ext[0] else None, n='COL(c)' if ext[1] else None)
+        idx = self._in_index(A, i, t='0', m='ROWC(r)' if ext[0] else None, n='COLC(c)' if ext[1] else None)
+        val = self._col_guard(f'ldf<{dt}>({A.p(f"in{i}")}, {idx})') if ext[1] else f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
         return (f'  float x{i}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
-                f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) x{i}[r][c] = ldf<{dt}>({A.p(f"in{i}")}, {idx});\n')
+                f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) x{i}[r][c] = {val};\n')
+
+    def _col_guard(self, expr: str) -> str:
+        """`expr` for real columns, 0 for padding columns (its address uses COLC, the clamped column)."""
+        return f'((COL(c) < {self.N}) ? {expr} : 0.0f)' if self.pad else expr
+
+    def _col_if(self) -> str:
+        """Statement prefix that skips padding columns."""
+        return f'if (COL(c) < {self.N}) ' if self.pad else ''
 
     def _ck_index(self, chunk: str) -> str:
-        N = self.plan.N
-        return f'(((i64)(b * H + h) * nch + ({chunk})) * M + (row0 + r)) * {N} + COL(c)'
+        return f'(((i64)(b * H + h) * nch + ({chunk})) * M + (row0 + r)) * {self.NP} + COL(c)'
 
     # ------------------------------------------------------------------ fw
     def fw(self, save: bool = True) -> KernelSpec:
@@ -498,7 +548,7 @@ class Emitter:
         rfront = self._row_front([g])
         if rfront:
             g = g.extract('fw', g.outputs, cut=rfront)
-        fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
+        fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant, self.colmask, self._lane_prolog())
         used_in = [i for i in range(nin) if p.in_names[i] in used]
         src, MT = self._row_kernel_common(R, W)
         body = []
@@ -510,7 +560,7 @@ class Emitter:
                 self._stage_input(stg, A, i, MT)
         if rfront:
             fn_src = self._stage_row_front(stg, A, rfront, set(used), MT, 'fw_rowpre') + '\n' + fn_src
-        body.append(stg.decls() + stg.bases())
+        body.append(stg.decls() + stg.bases() + stg.zero_pads())
         for k in range(nout):
             body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
         for k in range(naux):
@@ -520,9 +570,10 @@ class Emitter:
             rr, cc = _dims(st_ext[k], R, C)
             dt = DT_CODE[plan.st_dtypes[k]]
             nm = f'st{k}'
+            ld = self._col_guard(f'ldf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + '
+                                 f'(i64)ROWC(r) * {A.s(nm, 2)} + (i64)COLC(c) * {A.s(nm, 3)})')
             body.append(f'  float S{k}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
-                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) S{k}[r][c] = ldf<{dt}>({A.p(nm)}, '
-                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)ROWC(r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)});\n')
+                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) S{k}[r][c] = {ld};\n')
         for i in used_in:
             if not self.tdep[i]:
                 body.append(self._load_const_input(A, i, R, C))
@@ -593,11 +644,11 @@ class Emitter:
             dt = DT_CODE[plan.st_dtypes[k]]
             nm = f'stT{k}'
             body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
-                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) stf<{dt}>({A.p(nm)}, '
+                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) {self._col_if()}stf<{dt}>({A.p(nm)}, '
                         f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, S{k}[r][c]); }}\n')
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) {kname}(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
-        source = PRELUDE + A.struct() + fn_src + '\n' + kernel
+        source = PRELUDE + A.struct() + self._row_macros() + fn_src + '\n' + kernel
         return KernelSpec(kname, source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
 
     # ------------------------------------------------------------------ bw1
@@ -623,12 +674,12 @@ class Emitter:
         if rfront:
             g = g.extract('dstep', g.outputs, cut=rfront)
             restep_g = restep_g.extract('restep', restep_g.outputs, cut=rfront)
-        fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant)
+        fn_src, used = emit_graph_fn(g, 'bw_dstep', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant, self.colmask, self._lane_prolog())
         fns = [fn_src]
         used_all = set(used)
         re_used = []
         if needs_state:
-            re_src, re_used = emit_graph_fn(restep_g, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>', self.invariant)
+            re_src, re_used = emit_graph_fn(restep_g, 'bw_restep', R, C, st_ext, f'grp_allreduce<{L}>', self.invariant, self.colmask, self._lane_prolog())
             fns.append(re_src)
             used_all |= set(re_used)
         used_in = [i for i in range(nin) if p.in_names[i] in used_all]
@@ -651,7 +702,7 @@ class Emitter:
                                            f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'), A.s(nm, 1))
         if rfront:
             fns.insert(0, self._stage_row_front(stg, A, rfront, used_all, MT, 'bw_rowpre'))
-        body.append(stg.decls() + stg.bases())
+        body.append(stg.decls() + stg.bases() + stg.zero_pads())
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
         for i in tdep_col:
@@ -663,9 +714,10 @@ class Emitter:
             rr, cc = _dims(st_ext[k], R, C)
             dt = DT_CODE[plan.st_dtypes[k]]
             nm = f'dstT{k}'
+            ld = self._col_guard(f'ldf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + '
+                                 f'(i64)ROWC(r) * {A.s(nm, 2)} + (i64)COLC(c) * {A.s(nm, 3)})')
             body.append(f'  float D{k}[{rr}][{cc}];\n#pragma unroll\n  for (int r = 0; r < {rr}; r++)\n'
-                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) D{k}[r][c] = ldf<{dt}>({A.p(nm)}, '
-                        f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)ROWC(r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)});\n')
+                        f'#pragma unroll\n  for (int c = 0; c < {cc}; c++) D{k}[r][c] = {ld};\n')
         for i in used_in:
             if not self.tdep[i]:
                 body.append(self._load_const_input(A, i, R, C))
@@ -775,7 +827,7 @@ class Emitter:
                 rr, cc = _dims(st_ext[k], R, C)
                 body.append(f'    float Sh{k}_0[{rr}][{cc}];\n#pragma unroll\n    for (int r = 0; r < {rr}; r++)\n'
                             f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = '
-                            f'((const float*){A.p(f"sck{k}")})[(((i64)(b * H + h) * nch + (t0 / {DT})) * M + ROWC(r)) * {N} + COL(c)];\n')
+                            f'((const float*){A.p(f"sck{k}")})[(((i64)(b * H + h) * nch + (t0 / {DT})) * M + ROWC(r)) * {self.NP} + COL(c)];\n')
             for tt in range(1, DT):
                 for k in range(nst):
                     rr, cc = _dims(st_ext[k], R, C)
@@ -822,17 +874,17 @@ class Emitter:
             put = (f'atomic_addf({A.p(nm)}, {idx}, gmacc{i}[r][c])' if (bB or bH)
                    else f'stf<0>({A.p(nm)}, {idx}, gmacc{i}[r][c])')
             body.append(f'#pragma unroll\n  for (int r = 0; r < {R}; r++) if (row0 + r < M) {{\n#pragma unroll\n'
-                        f'    for (int c = 0; c < {C}; c++) {put}; }}\n')
+                        f'    for (int c = 0; c < {C}; c++) {self._col_if()}{put}; }}\n')
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
             dt = DT_CODE[plan.st_dtypes[k]]
             nm = f'dst{k}'
             body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
-                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) stf<{dt}>({A.p(nm)}, '
+                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) {self._col_if()}stf<{dt}>({A.p(nm)}, '
                         f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, D{k}[r][c]); }}\n')
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw1(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
-        source = PRELUDE + A.struct() + '\n'.join(fns) + '\n' + kernel
+        source = PRELUDE + A.struct() + self._row_macros() + '\n'.join(fns) + '\n' + kernel
         return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
 
     # ------------------------------------------------------------------ bw2
@@ -840,9 +892,11 @@ class Emitter:
         """`waves_per_simd` > 0 asks the compiler to fit that many waves on a SIMD (fewer registers,
         possibly spills); the caller compares the outcomes."""
         p, plan, t = self.p, self.plan, self.tile
-        N, DT = plan.N, t.DT
+        N, DT = plan.NP, t.DT              # lanes cover the padded width; `nok` marks real columns
         IPB = max(1, 64 // N)
         NT = max(64, N)
+        nok = 'nok' if self.pad else ''
+        nok_prolog = f'const bool nok = (int)(threadIdx.x % {N}) < {plan.N};' if self.pad else ''
         HB = max(1, getattr(t, 'HB', 1))
         MS = max(1, getattr(t, 'MS', 1))
         MR = -(-plan.M // MS)               # rows per instance
@@ -892,7 +946,7 @@ class Emitter:
         epi_exts = [self.in_ext(i) for i in rs]
         epi_nodes = {n_.name for n_ in p.epi.nodes}
         epi_g = p.epi.extract('epi', p.epi.outputs, cut=[f for f in rfront if f in epi_nodes]) if rfront else p.epi
-        epi_src, epi_used = emit_graph_fn(epi_g, 'bw_epi', 1, 1, epi_exts, red)
+        epi_src, epi_used = emit_graph_fn(epi_g, 'bw_epi', 1, 1, epi_exts, red, (), nok, nok_prolog)
         loop_used = set(drow_used) | set(re_used)
         pre_src, pre_used = '', []
         cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
@@ -902,7 +956,7 @@ class Emitter:
         rpre_used = []
         if rfront:
             rpre_g = p.joint.extract('rowpre', rfront, cut=set(cuts))
-            rpre_src, rpre_used = emit_graph_fn(rpre_g, 'bw_rowpre', 1, 1, [self.jext[f] for f in rfront], red, self.invariant)
+            rpre_src, rpre_used = emit_graph_fn(rpre_g, 'bw_rowpre', 1, 1, [self.jext[f] for f in rfront], red, self.invariant, nok, nok_prolog)
             pre_src += '\n' + rpre_src
         all_used = loop_used | set(epi_used) | set(rpre_used)
 
@@ -931,6 +985,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                      '  if (mlo >= M) return;')
         b.append(f'''  const int tid = threadIdx.x;
   const int n = tid % {N};
+  const bool nok = n < {plan.N}; const int nc = min(n, {plan.N - 1});     // real column? / column clamped for addresses
+  (void)nok; (void)nc;
   const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
   const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T;
@@ -966,8 +1022,9 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             ext = self.in_ext(i)
             dt = DT_CODE[plan.in_dtypes[i]]
             idx = self._in_index(A, i, t=(tclamp(tt) if self.tdep[i] else '0'),
-                                 m=('m' if ext[0] else None), n=('n' if ext[1] else None))
-            return f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
+                                 m=('m' if ext[0] else None), n=('nc' if ext[1] else None))
+            ld = f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
+            return f'(nok ? {ld} : 0.0f)' if (self.pad and ext[1]) else ld
 
         def var_in(i, tt):
             return f'x{i}_{tt}' if self.tdep[i] else f'x{i}'
@@ -1185,7 +1242,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for i in mats2:
             nmv = f'din{i}'
             idx = f'(i64)b * {A.s(nmv, 0)} + (i64)h * {A.s(nmv, 2)} + (i64)m * {A.s(nmv, 3)} + (i64)n * {A.s(nmv, 4)}'
-            b.append(f'    if (valid) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
+            b.append(f'    if (valid{" && nok" if self.pad else ""}) atomic_addf({A.p(nmv)}, {idx}, ma{i});\n')
         body = ''.join(b[body_start:])
         del b[body_start:]
         for j in range(PDe):
@@ -1203,7 +1260,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             nmv = f'din{i}'
             ext = self.in_ext(i)
             bB, bT, bH = bflags(i)
-            cond = 'valid' + ('' if ext[1] else ' && n == 0')
+            cond = 'valid' + ((' && nok' if self.pad else '') if ext[1] else ' && n == 0')
             if tail and not bT:
                 cond += f' && t0 + {tt} < T'
             idx = out_index(i, tt, hexpr)
@@ -1227,7 +1284,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append(f'  __shared__ float red_ms[{len(nred) * DT}][{NW}];\n')
             for q, j in enumerate(nred):
                 for tt in range(DT):
-                    b.append(f'  acc{j}_{tt} = grp_allreduce<64>(acc{j}_{tt});\n')
+                    b.append(f'  acc{j}_{tt} = grp_allreduce<64>({f"nok ? acc{j}_{tt} : 0.0f" if self.pad else f"acc{j}_{tt}"});\n')
             b.append('  __syncthreads();\n  if ((tid & 63) == 0) {\n')
             for q, j in enumerate(nred):
                 for tt in range(DT):
@@ -1242,7 +1299,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                 node = nm_[mname]
                 opext = self.jext[node.args[0]]
                 if 1 in node.dims and opext[1] and not batched:
-                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}(acc{j}_{tt});\n')
+                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}({f"nok ? acc{j}_{tt} : 0.0f" if self.pad else f"acc{j}_{tt}"});\n')
                 elif j in colsum:
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = s_cs{j}[inst][{tt}];\n')
                 else:

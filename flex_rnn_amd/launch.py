@@ -258,7 +258,7 @@ class CompiledPlan:
     def forward(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
-        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
+        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.NP          # (hidden buffers have the padded width)
         outs = tuple(th.empty(B, T, H, M, dtype=dt, device=dev) for dt in pl.out_dtypes)
         stT = tuple(th.empty_like(s) for s in state0)
         sck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state0)
@@ -301,7 +301,7 @@ class CompiledPlan:
     def backward(self, doutput, dstateT, inputs, state_store, aux):
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
-        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
+        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.NP          # (hidden buffers have the padded width)
         atomic = set(pl.atomic)
         daux = th.empty(len(p.daux), B, H, T, M, dtype=th.float32, device=dev)
         dck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state_store) \

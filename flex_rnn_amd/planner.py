@@ -106,6 +106,12 @@ class Plan:
     nchunks: int
 
     @property
+    def NP(self) -> int:
+        """State width the kernels are laid out for: N rounded up to a power of two.  The columns
+        beyond N are padding: never loaded or stored, masked out of every sum."""
+        return 1 << (self.N - 1).bit_length()
+
+    @property
     def atomic(self) -> List[int]:
         split = set(self.part.row_idx + self.part.scalar_idx) if self.tile.MS > 1 else set()
         return [i for i, b in enumerate(self.in_bcast) if any(b) or i in split]
@@ -147,7 +153,7 @@ def classify(inputs, state):
 
 def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
-    assert _is_pow2(N), f'state width N={N} must be a power of two (the state height M may be any size)'
+    N = 1 << (N - 1).bit_length()          # lanes and tiles cover the padded width
     nst = part.nstates + len(part.mat_idx)
 
     n_row = sum(1 for i in part.row_idx if in_bcast is None or not in_bcast[i][1])
@@ -281,7 +287,7 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
         if override:
             import dataclasses
             tile = dataclasses.replace(tile, **{k: int(v) for k, v in (kv.split('=') for kv in override.split(','))})
-    check_tile(tile, H, N, part)
+    check_tile(tile, H, 1 << (N - 1).bit_length(), part)
     nchunks = -(-T // tile.DT)
     plan = Plan(B, T, H, M, N, part, cls, [i.dtype for i in inputs], bcast,
                 [s.dtype for s in state], [o.dtype for o in output_t], tile, nchunks)
@@ -289,7 +295,7 @@ def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) 
     dev = 'meta'
     output_out = tuple(th.empty(B, T, H, M, dtype=o.dtype, device=dev) for o in output_t)
     dstate = tuple(th.empty_like(s, device=dev) for s in state)
-    state_store = tuple(th.empty(B, H, nchunks, M, N, dtype=th.float32, device=dev) for _ in state)
+    state_store = tuple(th.empty(B, H, nchunks, M, plan.NP, dtype=th.float32, device=dev) for _ in state)
     aux_out = (th.empty(len(part.aux), B, H, T, M, dtype=th.float32, device=dev),)
     dinputs_out = tuple(th.empty_like(i, device=dev) for i in inputs)
     forward_meta = get_meta([*output_out, *dstate, *state_store, *aux_out])

@@ -45,6 +45,14 @@ RUNS = [
     ('gla', '2,8,2,100,32', 'f32', 1),
     ('zoo', '1,8,2,5,8', 'f64', 0),
     ('gla', '1,8,2,16,16', 'f16', 1),
+    # state widths that are not a power of two (padding columns: masked sums, guarded loads / stores)
+    ('cfg:rwkv7', '1,16,2,24,96', 'f32', 0),
+    ('cfg:mamba1', '2,16,2,8,12', 'f32', 1),
+    ('cfg:mamba2', '2,16,2,8,160', 'bf16', 1),
+    ('cfg:gated_delta_rule', '1,16,2,16,80', 'f32', 0),
+    ('zoo2', '1,8,2,4,3', 'f32', 1),
+    ('s4d', '2,8,1,8,6', 'f32', 0),
+    ('delta_rule_fused', '2,16,2,8,20', 'f32', 1),
     # a single state row (M = 1), down to a scalar state (M = N = 1)
     ('mlstm_gates', '2,8,2,1,1', 'f32', 1),
     ('gla', '2,8,2,1,16', 'f32', 0),
@@ -105,6 +113,6 @@ def test_random_broadcast_patterns(seed):
 @pytest.mark.parametrize('seed', range(100, 112))
 def test_random_recurrences(seed):
     """Random step functions (tests/cases.py: random_step) through the emitted kernels."""
-    dims = ['2,8,2,8,16', '1,19,2,5,32', '2,16,1,24,128'][seed % 3]
+    dims = ['2,8,2,8,16', '1,19,2,5,32', '2,16,1,24,128', '2,8,2,8,24', '1,19,2,5,48', '2,16,1,12,5'][seed % 6]
     r = subprocess.run([sys.executable, RUNNER, f'gen:{seed}', dims, 'f32', str(seed % 2), '1e-4'], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2500:]}\n{r.stderr[-3000:]}'

@@ -193,7 +193,9 @@ def test_check_grad_and_benchmark_helpers():
                                        ('retention', (1, 32, 2, 16, 64)), ('mlstm_cell', (1, 32, 2, 32, 32)),
                                        ('zoo', (2, 32, 2, 32, 32)), ('zoo2', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
                                        # pointwise preparation inside the step: log-decay, in-step normalisation
-                                       ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32))])
+                                       ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32)),
+                                       # state widths that are not a power of two
+                                       ('rwkv7', (2, 32, 2, 64, 96)), ('mamba', (2, 32, 2, 32, 12)), ('gla', (1, 32, 2, 16, 160))])
 def test_other_recurrences(name, dims):
     print(f'case {name} {dims}', flush=True)
     step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)

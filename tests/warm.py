@@ -19,7 +19,8 @@ OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn'
          ('gla', (1, 32, 1, 16, 16)), ('delta_rule', (2, 32, 2, 16, 16)), ('gated_delta_rule', (2, 32, 2, 16, 16)),
          ('zoo', (2, 32, 2, 32, 32)), ('zoo2', (2, 32, 2, 32, 32)), ('gla', (2, 32, 2, 100, 32)),
          ('gla', (1, 16, 2, 16, 16)), ('gla', (3, 50, 2, 16, 16)), ('gla', (2, 33, 2, 16, 16)),
-         ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32))]
+         ('rwkv7', (2, 32, 2, 64, 64)), ('delta_rule_fused', (2, 32, 2, 32, 32)),
+         ('rwkv7', (2, 32, 2, 64, 96)), ('mamba', (2, 32, 2, 32, 12)), ('gla', (1, 32, 2, 16, 160))]
 
 
 EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
