@@ -9,6 +9,7 @@
 // PROT_NONE guard page, so an out-of-bounds access ends the process with SIGSEGV instead of
 // passing silently.
 #pragma once
+#define FRNN_HOST_HARNESS 1
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
