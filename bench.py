@@ -148,7 +148,7 @@ def main():
         'roofline': roofline, 'cpu_baseline': cpu,
         'gpu_kernel_ms_per_step': round(gpu_ms, 4),
         # candidate builds of the gradient kernel as timed on the first backward call (the fastest runs)
-        'row_kernel_builds': {k: {'rows_per_lane, waves': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
+        'row_kernel_builds': {k: {'tiles (L, C, R, W)': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
                                   'ms': compiled.build_times.get(k) and [round(v, 4) for v in compiled.build_times[k]]}
                               for k in ('frnn_fw', 'frnn_bw1')},
         'gradient_kernel_builds': [

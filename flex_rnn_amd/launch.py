@@ -91,18 +91,31 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
 
 
 def row_kernel_tiles(plan, reverse: bool):
-    """(R, W) candidates for the forward kernel (or the reverse scan): the heuristic's choice first,
-    then half the rows per lane (more, lighter waves) with the same and with twice the waves per
-    workgroup.  Which is fastest depends on how many (batch, head) pairs there are, on the LDS
-    traffic of the staged operands and on register use; the first call times them."""
+    """(L, C, R, W) candidates for the forward kernel (or the reverse scan): the heuristic's choice
+    first; half the rows per lane (more, lighter waves) with the same and with twice the waves per
+    workgroup; and, where the heuristic spread a state row over more than one 16-lane DPP row to get
+    more waves, twice the columns per lane (cheaper reductions, fewer waves).  Which is fastest
+    depends on how many (batch, head) pairs there are, on the LDS traffic of the staged operands
+    and on register use; the first call times them."""
     t = plan.tile
     R, W = ((t.R1 or t.R), (t.W1 or t.W)) if reverse else (t.R, t.W)
-    G = t.G
-    out = [(R, W)]
     fixed_r = reverse and plan.part.dstep_needs_state          # one row per lane there (register budget)
-    for r, w in ((R // 2, W), (R // 2, 2 * W)) if (R > 1 and not fixed_r) else ((R, 2 * W),):
-        if r >= 1 and w <= 8 and w * G * r <= max(plan.M, G * r) and (r, w) not in out:
-            out.append((r, w))
+    out = []
+
+    def add(L, C, r, w):
+        G = 64 // L
+        if r >= 1 and 1 <= w <= 8 and (w == 1 or w * G * r <= max(plan.M, G * r)) and (L, C, r, w) not in out and len(out) < 5:
+            out.append((L, C, r, w))
+
+    add(t.L, t.C, R, W)
+    if R > 1 and not fixed_r:
+        add(t.L, t.C, R // 2, W)
+        add(t.L, t.C, R // 2, 2 * W)
+    else:
+        add(t.L, t.C, R, 2 * W)
+    if t.L > 16 and t.C < 8:
+        add(t.L // 2, t.C * 2, R, W)
+        add(t.L // 2, t.C * 2, R, 2 * W)
     return out
 
 
@@ -110,8 +123,9 @@ def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save:
     """[(spec, path)] for `row_kernel_tiles`, compiled side by side (`save=False`: the inference
     variant of the forward kernel)."""
     specs = []
-    for r, w in row_kernel_tiles(plan, reverse):
-        tile = dataclasses.replace(plan.tile, R1=r, W1=w) if reverse else dataclasses.replace(plan.tile, R=r, W=w)
+    for L, C, r, w in row_kernel_tiles(plan, reverse):
+        tile = dataclasses.replace(plan.tile, L=L, C=C)
+        tile = dataclasses.replace(tile, R1=r, W1=w) if reverse else dataclasses.replace(tile, R=r, W=w)
         em = Emitter(dataclasses.replace(plan, tile=tile))
         specs.append(em.bw1() if reverse else em.fw(save=save))
     return _compile(specs, force, seen)
