@@ -231,8 +231,10 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     # (measured: where splitting would turn plain stores of row gradients into atomics - RWKV-7 at a
     # small batch - it costs more than the extra waves bring; with inputs shared over batch, time or
     # heads the gradients are accumulated atomically anyway - Mamba-1 - and it pays)
-    if part.epi_linear and shared:
-        while waves2 * MS < 32 * 4 * n_cu and -(-M // (2 * MS)) >= 8:
+    # Otherwise rows are only split when the chip would be mostly idle (under two waves per SIMD).
+    if part.epi_linear:
+        target = (32 if shared else 2) * 4 * n_cu
+        while waves2 * MS < target and -(-M // (2 * MS)) >= 8:
             MS *= 2
     return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, R1=R1, W1=W1, HB=1, MS=MS)
 
