@@ -87,7 +87,20 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
         return (0 if res['scratch'] <= MAX_SPILL_BYTES else 1, -res['occupancy'], res['scratch'])
 
     order = sorted(range(len(cands)), key=lambda i: (rank(cands[i]), i))
-    return [cands[i] for i in order]
+    ranked = [cands[i] for i in order]
+    # with split rows (every build then accumulates atomically into the same fp32 buffers), the
+    # first-ranked build also with a quarter and with four times as many splits
+    ms = plan.tile.MS
+    if ms > 1:
+        top = ranked[0][0].source
+        wps = int(top.split('amdgpu_waves_per_eu(')[1].split(',')[0]) if 'amdgpu_waves_per_eu(' in top else 0
+        first = len(cands)
+        for alt in (ms // 4, ms * 4):
+            if alt >= 2 and -(-plan.M // alt) >= 4 and alt <= 65535:
+                em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
+                add([em_alt.bw2(waves_per_simd=wps, prefetch=4)])
+        ranked += cands[first:]
+    return ranked
 
 
 def row_kernel_tiles(plan, reverse: bool):

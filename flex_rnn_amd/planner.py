@@ -233,7 +233,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     # heads the gradients are accumulated atomically anyway - Mamba-1 - and it pays)
     # Otherwise rows are only split when the chip would be mostly idle (under two waves per SIMD).
     if part.epi_linear:
-        target = (32 if shared else 2) * 4 * n_cu
+        target = (32 if (shared or N <= 32) else 2) * 4 * n_cu      # (narrow states: light instances, several per wave)
         while waves2 * MS < target and -(-M // (2 * MS)) >= 8:
             MS *= 2
     return TileConfig(L=L, C=C, R=R, W=W, DT=DT, TS=TS, R1=R1, W1=W1, HB=1, MS=MS)
