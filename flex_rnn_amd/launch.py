@@ -44,9 +44,19 @@ def _compile(specs, force, seen):
             seen.add(key)
         jobs.append((s, again))
     # independent compiler processes: wait for them side by side (the runtime call releases the GIL)
+    def one(j):
+        try:
+            return runtime.compile_kernel(j[0].name, j[0].source, force=j[1])
+        except runtime.RuntimeError_ as e:
+            return e
+
     with ThreadPoolExecutor(max_workers=max(1, len(jobs))) as pool:
-        paths = list(pool.map(lambda j: runtime.compile_kernel(j[0].name, j[0].source, force=j[1]), jobs))
-    return [(s, path) for (s, _), path in zip(jobs, paths)]
+        paths = list(pool.map(one, jobs))
+    # the first spec is the one the caller cannot do without; a further candidate that does not
+    # build (e.g. a tile whose staging exceeds the LDS limit) is dropped
+    if paths and isinstance(paths[0], Exception):
+        raise paths[0]
+    return [(s, path) for (s, _), path in zip(jobs, paths) if not isinstance(path, Exception)]
 
 
 def gradient_kernel_builds(plan, force: bool = False, seen=None):
@@ -63,10 +73,16 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
     em = Emitter(plan)
     cands, seen_src = [], set()
 
-    def add(specs):
+    def add(specs, optional=False):
         specs = [sp for sp in specs if sp.source not in seen_src and not seen_src.add(sp.source)]
         out = []
-        for spec, path in _compile(specs, force, seen):
+        try:
+            built = _compile(specs, force, seen)
+        except runtime.RuntimeError_:
+            if not optional:
+                raise
+            built = []
+        for spec, path in built:
             res = runtime.kernel_resources(path)
             cands.append((spec, path, res))
             out.append(res)
@@ -78,7 +94,7 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
     for pd, res in zip(depths, plain):          # (a duplicate source was dropped: zip stops short, which is fine)
         if res is not None and res['occupancy'] < 4 and (res['occupancy'] < 2 or res['vgprs'] <= 224):
             more.append(em.bw2(waves_per_simd=res['occupancy'] + 1, prefetch=pd))
-    add(more)
+    add(more, optional=True)
 
     def rank(c):
         res = c[2]
@@ -98,7 +114,7 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
         for alt in (ms // 4, ms * 4):
             if alt >= 2 and -(-plan.M // alt) >= 4 and alt <= 65535:
                 em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
-                add([em_alt.bw2(waves_per_simd=wps, prefetch=4)])
+                add([em_alt.bw2(waves_per_simd=wps, prefetch=4)], optional=True)
         ranked += cands[first:]
     return ranked
 
@@ -266,15 +282,20 @@ class CompiledPlan:
         times = []
         for i in range(len(self.builds[name])):
             self._select(name, i)
-            self._launch(name, tensors)
             best = float('inf')
-            for _ in range(2):
-                e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
-                e0.record()
+            try:
                 self._launch(name, tensors)
-                e1.record()
-                e1.synchronize()
-                best = min(best, e0.elapsed_time(e1))
+                for _ in range(2):
+                    e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
+                    e0.record()
+                    self._launch(name, tensors)
+                    e1.record()
+                    e1.synchronize()
+                    best = min(best, e0.elapsed_time(e1))
+            except runtime.RuntimeError_:
+                if i == 0:
+                    raise                       # the first-ranked build must be launchable
+                best = float('inf')             # (a candidate the device refuses to launch is just not taken)
             times.append(best)
         self._select(name, min(range(len(times)), key=times.__getitem__))
         self.build_times[name] = times
