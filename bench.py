@@ -30,6 +30,12 @@ WORK = {
 }
 
 
+# The only published figure for the headline metric: the reference's README (lines 52-75), RWKV-7 B8 T1024 H32
+# 128x128 bf16 fwd+bwd, 55 ms per step on an RTX 4070 mobile = 8192 tokens / 55 ms.  Other hardware: context only.
+PUBLISHED_TOKENS_PER_S = {'rwkv7': 8192 / 55e-3}
+PUBLISHED_NOTE = 'reference README: 55 ms per fwd+bwd step on an RTX 4070 mobile (other hardware)'
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -42,7 +48,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print(f'bench.py: this build measures one GPU; --gpus {args.gpus} is not supported '
-              '(the recurrence shards over batch x head with no exchange, see DESIGN.md).', file=sys.stderr)
+              '(the recurrence shards over batch x head with no exchange between GPUs; each GPU would run this same path).', file=sys.stderr)
         sys.exit(2)
 
     import torch as th
@@ -142,7 +148,10 @@ def main():
     out = {
         'metric': 'fwd+bwd tokens/sec', 'value': round(value, 1), 'unit': 'tokens/s', 'n_gpus': 1,
         'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
-        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f32',
+        'higher_is_better': True, 'scaling': 'weak',
+        'vs_baseline': round(value / PUBLISHED_TOKENS_PER_S[name], 2) if name in PUBLISHED_TOKENS_PER_S else None,
+        'baseline_note': PUBLISHED_NOTE if name in PUBLISHED_TOKENS_PER_S else None,
+        'dtype': 'f32',
         'io_dtype': str(wl.dtype).replace('torch.', ''), 'data': 'synthetic',
         'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
         'roofline': roofline, 'cpu_baseline': cpu,
