@@ -93,7 +93,7 @@ class jit:
                 fwd = self.forward_func
             return fwd.forward_only(inputs, state)
 
-    # ------------------------------------------------------------------ oracle
+    # ------------------------------------------------------------------ plain per-timestep loop
     def naive(self, *args, dtype=th.float32):
         """Pure-PyTorch per-timestep loop with the compiled path's calling convention
         (jit.py:23-36): inputs are cast to `dtype`, the initial state is not; outputs

@@ -58,11 +58,18 @@ class SimPlan(CompiledPlan):
         self.against_end = against_end
         self.kernels = {}
         # HIPSIM_PREFETCH selects the gradient kernel's variant with that many checkpoint rows in flight
-        for spec in kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4'))):
+        specs = kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4')))
+        from flex_rnn_amd.emit_hip import Emitter
+        specs.append(Emitter(plan).fw(save=False))          # the inference kernel, used by forward_only()
+        from concurrent.futures import ThreadPoolExecutor
+        with ThreadPoolExecutor(max_workers=len(specs)) as pool:      # host compiler runs side by side
+            list(pool.map(_compile_host, specs))
+        for spec in specs:
             self._add_kernel(spec)
 
     def _add_builds(self, name, built):
-        self._add_kernel(built[0][0])
+        if name not in self.kernels:
+            self._add_kernel(built[0][0])
 
     def _tune(self, name, tensors, accumulators=()):
         pass

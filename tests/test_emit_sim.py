@@ -14,13 +14,10 @@ RUNNER = os.path.join(HERE, 'hipsim', 'run_case.py')
 # (case, B,T,H,M,N, dtype, guard at end?)
 RUNS = [
     ('cfg:delta_rule', '1,64,2,16,16', 'f32', 1),
-    ('cfg:delta_rule', '1,64,2,16,16', 'f32', 0),
     ('cfg:mamba1', '2,16,2,128,16', 'f32', 1),      # reverse scan with state recompute, matrix grads, atomics
-    ('cfg:mamba1', '2,16,2,128,16', 'f32', 0),
-    ('cfg:mamba2', '2,16,2,64,128', 'bf16', 1),     # scalar inputs, head-broadcast rows
-    ('cfg:rwkv7', '1,16,2,128,128', 'bf16', 1),
-    ('cfg:rwkv7', '1,16,2,128,128', 'f32', 0),
-    ('cfg:gated_delta_rule', '1,16,2,128,128', 'bf16', 1),
+    ('cfg:mamba2', '1,16,2,64,128', 'bf16', 1),     # scalar inputs, head-broadcast rows
+    ('cfg:rwkv7', '1,16,1,128,128', 'bf16', 1),
+    ('cfg:gated_delta_rule', '1,16,1,128,128', 'bf16', 1),
     ('rwkv7', '1,16,2,64,64', 'bf16', 0),           # log-decay: exp evaluated while staging / once per chunk
     ('delta_rule_fused', '2,16,2,16,32', 'f32', 1), # in-step normalisation (row-only sum) and gate
     ('rwkv6', '2,8,2,16,16', 'f32', 1),             # time-independent row input
@@ -32,9 +29,9 @@ RUNS = [
     ('rwkv4', '2,8,1,32,1', 'f32', 0),              # three states, comparisons
     ('mlstm_gates', '2,8,2,16,1', 'f32', 1),        # three outputs
     # sequence lengths that are not a multiple of the chunk (partial last chunk), and T = 1
-    ('cfg:rwkv7', '1,37,2,128,128', 'f32', 0),
+    ('cfg:rwkv7', '1,37,1,128,128', 'f32', 0),
     ('cfg:mamba1', '2,13,2,128,16', 'f32', 1),
-    ('cfg:mamba2', '2,21,2,64,128', 'bf16', 0),
+    ('cfg:mamba2', '1,21,2,64,128', 'bf16', 0),
     ('rwkv4', '2,11,1,32,1', 'f32', 0),
     ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1),
     # the emitter's op table (sigmoid, tanh, softplus, where, relu, sqrt, rsqrt, log, min/max, ...)
@@ -74,8 +71,8 @@ TILED = [
     ('cfg:mamba2', '2,16,4,16,128', 'f32', 0, 'HB=2,MS=1'),
     ('cfg:mamba2', '2,16,4,16,128', 'f32', 1, 'HB=4,MS=2'),
     # row-kernel tiles that the first-call timing may pick instead of the heuristic's
-    ('cfg:rwkv7', '1,16,2,128,128', 'f32', 0, 'R=2,W=8,R1=2,W1=4'),
-    ('cfg:mamba2', '2,16,2,64,128', 'f32', 1, 'R=1,W=8,R1=1,W1=8'),
+    ('cfg:rwkv7', '1,16,1,128,128', 'f32', 0, 'R=2,W=8,R1=2,W1=4'),
+    ('cfg:mamba2', '1,16,2,64,128', 'f32', 1, 'R=1,W=8,R1=1,W1=8'),
     ('cfg:mamba1', '2,16,2,128,16', 'f32', 0, 'R=1,W=8,R1=1,W1=8'),
 ]
 
@@ -103,14 +100,14 @@ def _random_pattern_case(seed):
     return 'pattern:' + ','.join(spans)
 
 
-@pytest.mark.parametrize('seed', range(6))
+@pytest.mark.parametrize('seed', range(4))
 def test_random_broadcast_patterns(seed):
     case = _random_pattern_case(seed)
     r = subprocess.run([sys.executable, RUNNER, case, '2,8,3,8,16', 'f32', str(seed % 2)], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'{case}\nrc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
 
 
-@pytest.mark.parametrize('seed', range(100, 112))
+@pytest.mark.parametrize('seed', range(100, 106))
 def test_random_recurrences(seed):
     """Random step functions (tests/cases.py: random_step) through the emitted kernels."""
     dims = ['2,8,2,8,16', '1,19,2,5,32', '2,16,1,24,128', '2,8,2,8,24', '1,19,2,5,48', '2,16,1,12,5'][seed % 6]
