@@ -75,6 +75,29 @@ def test_chunked_call_equals_single_call_at_full_size():
     assert recurrence.rel_err(S2, S) < 1e-2
 
 
+@pytest.mark.parametrize('name', ['rwkv7', 'mamba2', 'mamba1', 'gated_delta_rule'])
+def test_backward_is_linear_in_upstream_gradients_at_full_size(name):
+    """Size-independent property at the benchmark sizes: the gradients for 0.5 * g1 - 2 * g2 are
+    0.5 * grads(g1) - 2 * grads(g2), for every input and the initial state (tolerance: the I/O dtype's
+    rounding of three separately rounded results)."""
+    print(f'case linear backward {name} full', flush=True)
+    wl = configs.make(name)
+    f = flex_rnn_amd.jit(wl.step)
+    xs = [x.requires_grad_() for x in _gpu(wl.inputs)]
+    ss = [s_.requires_grad_() for s_ in _gpu(wl.states)]
+    out = f(*xs, *ss)
+    gen = th.Generator(device='cuda').manual_seed(1)
+    g1 = [th.randn(o.shape, generator=gen, device='cuda').to(o.dtype) for o in out]
+    g2 = [th.randn(o.shape, generator=gen, device='cuda').to(o.dtype) for o in out]
+    mix = [(0.5 * a.float() - 2.0 * b.float()).to(a.dtype) for a, b in zip(g1, g2)]
+    r1 = th.autograd.grad(out, xs + ss, g1, retain_graph=True)
+    r2 = th.autograd.grad(out, xs + ss, g2, retain_graph=True)
+    rm = th.autograd.grad(out, xs + ss, mix)
+    tol = 2e-2 if wl.dtype == th.bfloat16 else 1e-4
+    for a, b, m in zip(r1, r2, rm):
+        assert recurrence.rel_err(m, 0.5 * a.double() - 2.0 * b.double()) < tol
+
+
 def test_strided_and_broadcast_views_match_contiguous_copies():
     """The adapter pattern of the reference's examples: [B,T,H,C] tensors unsqueezed, `v.mT`
     and a transposed state, plus an expanded (stride-0) input; no copies are made."""
