@@ -10,6 +10,7 @@ fp32 scratch + cast-back for gradients of inputs broadcast over batch / time / h
 """
 from __future__ import annotations
 
+import contextlib
 import dataclasses
 import os
 import struct
@@ -176,8 +177,10 @@ def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec,
 class CompiledPlan:
     _tune_pending = frozenset()
 
-    def __init__(self, plan, state_meta=None):
+    def __init__(self, plan, state_meta=None, device=None):
         self.plan = plan
+        # code objects are loaded for one device; tensors of later calls must live there
+        self.device = th.device(device) if device is not None else None
         # (shape, stride, dtype) of the initial states: gradients w.r.t. them are laid out alike
         self.state_meta = state_meta
         # when set to a list, every launch appends (kernel name, start event, end event)
@@ -209,7 +212,9 @@ class CompiledPlan:
             if needs_gradient_kernel(plan.part):
                 jobs['frnn_bw2'] = pool.submit(gradient_kernel_builds, plan)
             built = {k: j.result() for k, j in jobs.items()}
-        self.builds = {k: [(s_, load(s_, p_), r_) for s_, p_, r_ in v] for k, v in built.items()}
+        on_gpu = self.device is not None and self.device.type == 'cuda'
+        with (th.cuda.device(self.device) if on_gpu else contextlib.nullcontext()):
+            self.builds = {k: [(s_, load(s_, p_), r_) for s_, p_, r_ in v] for k, v in built.items()}
         self.build_times = {}
         tune = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
         self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1}
@@ -237,7 +242,9 @@ class CompiledPlan:
         self._packer[name] = struct.Struct('<' + 'q5q' * max(len(spec.tensors), 1) + '5q')
 
     def _add_builds(self, name, built):
-        self.builds[name] = [(s_, self._load(s_, p_), r_) for s_, p_, r_ in built]
+        on_gpu = self.device is not None and self.device.type == 'cuda'
+        with (th.cuda.device(self.device) if on_gpu else contextlib.nullcontext()):
+            self.builds[name] = [(s_, self._load(s_, p_), r_) for s_, p_, r_ in built]
         if len(built) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0':
             self._tune_pending.add(name)
         self._select(name, 0)
@@ -253,6 +260,8 @@ class CompiledPlan:
             assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
             dev = t.device if dev is None else dev
             assert t.device == dev, 'all tensors must live on the same device'
+            assert self.device is None or t.device == self.device, \
+                f'this instance was compiled for {self.device}; got a tensor on {t.device}'
             vals.append(t.data_ptr())
             vals.extend(_strides5(t))
         if not spec.tensors:

@@ -317,7 +317,8 @@ def build_twopass(step: Callable, inputs, state, dryrun: bool = False, tile: Opt
         return forward_meta, backward_meta
 
     from .launch import CompiledPlan
-    compiled = CompiledPlan(plan, state_meta=forward_meta[plan.part.noutputs:plan.part.noutputs + plan.part.nstates])
+    compiled = CompiledPlan(plan, state_meta=forward_meta[plan.part.noutputs:plan.part.noutputs + plan.part.nstates],
+                            device=inputs[0].device)
 
     in_meta = tuple(th.empty_strided(i.shape, i.stride(), dtype=i.dtype, device='meta') for i in inputs)
     st_meta = tuple(th.empty_strided(s.shape, s.stride(), dtype=s.dtype, device='meta') for s in state)
