@@ -69,7 +69,7 @@ def test_chunked_call_equals_single_call_at_full_size():
     y1, S1 = g(*[x[:, :T // 2] for x in xs], *ss)
     h = flex_rnn_amd.jit(wl.step)
     y2, S2 = h(*[x[:, T // 2:] for x in xs], S1)
-    assert th.equal(y1, y[:, :T // 2])
+    assert recurrence.rel_err(y1, y[:, :T // 2]) < 1e-3      # (equal unless the first-call timing picked other tiles)
     # the hand-off state passes through bf16 storage once more than inside a single call
     assert recurrence.rel_err(y2, y[:, T // 2:]) < 1e-2
     assert recurrence.rel_err(S2, S) < 1e-2
@@ -174,7 +174,10 @@ def test_infer_matches_call(name):
     xs, ss = _gpu(wl.inputs), _gpu(wl.states)
     a = f.infer(*xs, *ss)
     b = f(*xs, *ss)
-    assert len(a) == len(b) and all(th.equal(x, y) for x, y in zip(a, b))
+    # (the two kernels may have been given different tiles by the first-call timing, hence a
+    # different order of the additions inside a row sum: equal up to rounding of the I/O dtype)
+    tol = 1e-2 if wl.dtype == th.bfloat16 else 1e-5
+    assert len(a) == len(b) and all(recurrence.rel_err(x, y) < tol for x, y in zip(a, b))
     assert not any(t.requires_grad for t in a)
 
 

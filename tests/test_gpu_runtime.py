@@ -97,9 +97,10 @@ def test_corrupt_cache_entry_is_rebuilt(tmp_path, monkeypatch):
     S = th.zeros(1, 1, 16, 16).cuda()
     y0, _ = flex_rnn_amd.jit(ops.gla)(q, k, v, gate, S)          # fills the cache
     files = glob.glob(os.path.join(str(tmp_path), 'frnn_fw_*.hsaco'))
-    assert len(files) == 1
-    with open(files[0], 'wb') as f:
-        f.write(b'not a code object')
+    assert len(files) >= 1                                      # (one per candidate tile)
+    for path in files:
+        with open(path, 'wb') as f:
+            f.write(b'not a code object')
     y1, _ = flex_rnn_amd.jit(ops.gla)(q, k, v, gate, S)          # new instance: loads from the cache
     th.cuda.synchronize()
-    assert th.equal(y0, y1) and os.path.getsize(files[0]) > 1000
+    assert (y0 - y1).abs().max().item() < 1e-5 and all(os.path.getsize(p_) > 1000 for p_ in files)
