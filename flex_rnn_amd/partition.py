@@ -26,7 +26,7 @@ and saved when `drow` needs them.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Sequence, Tuple
+from typing import Dict, List, Sequence
 
 from .ir import Graph
 
@@ -107,10 +107,6 @@ def _linear_in(graph: Graph, seeds: Sequence[str]) -> bool:
             r = NON
         kind[n.name] = r
     return all(kind[o] == LIN for o in graph.outputs)
-
-
-def classify_index(ext: Tuple[bool, bool]) -> str:
-    return {(True, True): 'mat', (True, False): 'col', (False, True): 'row', (False, False): 'scalar'}[ext]
 
 
 def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
