@@ -24,6 +24,7 @@ cache key, which is a hash of the source).
 from __future__ import annotations
 
 import math
+import os
 from dataclasses import dataclass
 from typing import List, Sequence, Tuple
 
@@ -31,6 +32,8 @@ import torch as th
 
 from .ir import Graph
 
+# blocks a launch may have along grid y (hardware limit; the variable lets a test reach the folded form at small sizes)
+MAX_GRID_Y = int(os.environ.get('FLEX_RNN_MAX_GRID_Y', '65535'))
 DT_CODE = {th.float32: 0, th.bfloat16: 1, th.float16: 2, th.float64: 3}
 
 PRELUDE = r'''
@@ -1001,6 +1004,12 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         rows_decl = ('  const int mlo = 0, mhi = M;' if MS == 1 else
                      f'  const int mlo = blockIdx.z * {MR}, mhi = min(M, mlo + {MR});   // rows of this instance\n'
                      '  if (mlo >= M) return;')
+        # grid y is limited to 65535 blocks: with more (batch, head group) pairs than that, both indices
+        # travel in x, in the same order of dispatch
+        fold = plan.B * (plan.H // HB) > MAX_GRID_Y
+        block_decl = (f'  const int gx_ = (nch + {IPB - 1}) / {IPB};\n  const int bx_ = blockIdx.x % gx_, by_ = blockIdx.x / gx_;\n'
+                      if fold else '')
+        bx, by = ('bx_', 'by_') if fold else ('blockIdx.x', 'blockIdx.y')
         b.append(f'''  const int tid = threadIdx.x;
   const int n = tid % {N};
   const bool nok = n < {plan.N}; const int nc = min(n, {plan.N - 1});     // real column? / column clamped for addresses
@@ -1008,11 +1017,11 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
   const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T;
-  int ch = blockIdx.x * {IPB} + inst;
+{block_decl}  int ch = {bx} * {IPB} + inst;
   const bool valid = ch < nch;
   if (!valid) ch = nch - 1;
   const int HG = H / {HB};                     // head groups; an instance walks {HB} heads
-  const int b = blockIdx.y / HG, h0 = (blockIdx.y % HG) * {HB};
+  const int b = {by} / HG, h0 = ({by} % HG) * {HB};
   const int t0 = ch * {DT};
 {rows_decl}
   const int nt = {f"min({DT}, T - t0)" if self.tail_dt else DT};          // timesteps of this chunk
@@ -1351,4 +1360,5 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         attr = f' __attribute__((amdgpu_waves_per_eu({wpe},{wpe})))' if wpe else ''
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){attr} frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
         source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + pre_src + '\n' + kernel
-        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})', str(MS)))
+        gx, gy = f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})'
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'({gx}) * {gy}', '1', str(MS)) if fold else (gx, gy, str(MS)))

@@ -86,6 +86,14 @@ def test_tile_overrides(case, dims, dtype, end, tile):
     assert tile.split(',')[0] in r.stdout.replace(' ', '')
 
 
+@pytest.mark.parametrize('case,dims', [('rwkv7', '3,32,2,16,16'), ('cfg:mamba1', '2,16,4,32,16')])
+def test_more_batch_head_pairs_than_grid_y_allows(case, dims):
+    """The gradient kernel then carries both block indices in grid x (limit lowered to 3 so that small sizes reach it)."""
+    env = dict(os.environ, FLEX_RNN_MAX_GRID_Y='3')
+    r = subprocess.run([sys.executable, RUNNER, case, dims, 'f32', '1'], capture_output=True, text=True, timeout=900, env=env)
+    assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
+
+
 def _random_pattern_case(seed):
     """A gated linear-attention step whose five inputs get random classes-compatible broadcast
     patterns over (B, T, H); returns the argument string of run_case.py's `pattern:` mode."""
