@@ -257,18 +257,20 @@ class CompiledPlan:
         dev = None
         for name in spec.tensors:
             t = tensors[name]
-            assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
-            dev = t.device if dev is None else dev
-            assert t.device == dev, 'all tensors must live on the same device'
-            assert self.device is None or t.device == self.device, \
-                f'this instance was compiled for {self.device}; got a tensor on {t.device}'
+            if t.device != dev:
+                assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
+                assert dev is None, 'all tensors must live on the same device'
+                assert self.device is None or t.device == self.device, \
+                    f'this instance was compiled for {self.device}; got a tensor on {t.device}'
+                dev = t.device
             vals.append(t.data_ptr())
             vals.extend(_strides5(t))
         if not spec.tensors:
             vals = [0] * 6
         buf = self._packer[kname].pack(*vals, pl.B, pl.T, pl.H, pl.M, pl.nchunks)
         grid = self._grid[kname]
-        with th.cuda.device(dev):
+        other = dev is not None and th.cuda.current_device() != dev.index
+        with (th.cuda.device(dev) if other or dev is None else contextlib.nullcontext()):
             stream = th.cuda.current_stream(dev).cuda_stream
             if self.profile_events is not None:
                 e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
@@ -367,12 +369,15 @@ class CompiledPlan:
             dst0 = tuple(th.empty_strided(sh, st, dtype=dt, device=dev) for sh, st, dt in self.state_meta)
         else:
             dst0 = tuple(th.empty_like(s) for s in dstateT)
-        dins = []
-        for i, x in enumerate(inputs):
-            if i in atomic:
-                dins.append(th.zeros(x.shape, dtype=th.float32, device=dev))
-            else:
-                dins.append(th.empty_like(x))
+        # Gradients that several workgroups add into accumulate in fp32.  Those of fp32 contiguous inputs are
+        # handed out as they are; the others share one zero-filled buffer and are cast at the end.
+        order = sorted(atomic)
+        cast = [i for i in order if inputs[i].dtype != th.float32 or not inputs[i].is_contiguous()]
+        sizes = [inputs[i].numel() for i in cast]
+        flat = th.zeros(sum(sizes), dtype=th.float32, device=dev).split(sizes) if cast else ()
+        scratch = {i: f.view(inputs[i].shape) for i, f in zip(cast, flat)}
+        dins = [scratch[i] if i in scratch else th.zeros_like(x) if i in atomic else th.empty_like(x)
+                for i, x in enumerate(inputs)]
         tensors = {'aux': aux, 'daux': daux}
         for i, x in enumerate(inputs):
             tensors[f'in{i}'] = x
@@ -385,15 +390,15 @@ class CompiledPlan:
                 tensors[f'dck{k}'] = dck[k]
         for k in range(p.noutputs):
             tensors[f'dout{k}'] = doutput[k]
-        acc = [dins[i] for i in atomic]             # zero so far; each kernel adds its own inputs' gradients
+        acc = [dins[i] for i in order]              # zero so far; each kernel adds its own inputs' gradients
         self._tune('frnn_bw1', tensors, acc)
         self._launch('frnn_bw1', tensors)
         if 'frnn_bw2' in self.kernels:
             self._tune('frnn_bw2', tensors, acc)
             self._launch('frnn_bw2', tensors)
-        for i in atomic:
-            x = inputs[i]
-            g = th.empty_like(x)
-            g.copy_(dins[i])
-            dins[i] = g
+        if cast:                                    # (to the inputs' dtype and layout)
+            final = [th.empty_like(inputs[i]) for i in cast]
+            th._foreach_copy_(final, [dins[i] for i in cast])
+            for i, g in zip(cast, final):
+                dins[i] = g
         return tuple(dins), dst0

@@ -162,6 +162,9 @@ def kernel_resources(hsaco: str):
         return None
 
 
+_U3 = ctypes.c_uint32 * 3
+
+
 class Kernel:
     def __init__(self, module: 'Module', name: str):
         self.module = module
@@ -171,10 +174,9 @@ class Kernel:
         self.handle = h
 
     def launch(self, grid: Sequence[int], block: Sequence[int], args: bytes, stream: int = 0, lds_bytes: int = 0):
-        g = (ctypes.c_uint32 * 3)(*grid)
-        b = (ctypes.c_uint32 * 3)(*block)
-        buf = ctypes.create_string_buffer(args, len(args))
-        _check(lib().frnn_launch(self.handle, g, b, lds_bytes, ctypes.c_void_p(stream), buf, len(args)),
+        g = _U3(*grid)
+        b = _U3(*block)
+        _check(lib().frnn_launch(self.handle, g, b, lds_bytes, ctypes.c_void_p(stream), args, len(args)),
                f'launching kernel {self.name}')
 
 
