@@ -155,3 +155,15 @@ def random_step(seed):
     env = {'th': th, 'F': F}
     exec(src, env)
     return env['step'], spec, 1, src
+
+
+# Random recurrences that run both through the emitted kernels on the CPU harness and on the GPU:
+# seed -> B, T, H, M, N (widths that are no power of two included)
+FUZZ_DIMS = [(2, 8, 2, 8, 16), (1, 19, 2, 5, 32), (2, 16, 1, 24, 128), (2, 8, 2, 8, 24), (1, 19, 2, 5, 48), (2, 16, 1, 12, 5)]
+FUZZ_SEEDS = range(100, 112)
+
+
+def fuzz_case(seed, dtype):
+    """(step, inputs, states) of random recurrence `seed` at its size in FUZZ_DIMS."""
+    step, spec, nst, _ = random_step(seed)
+    return make_inputs('gen', *FUZZ_DIMS[seed % 6], dtype=dtype, table={'gen': (step, spec, nst)})

@@ -8,6 +8,8 @@ import sys
 
 import pytest
 
+import cases
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 RUNNER = os.path.join(HERE, 'hipsim', 'run_case.py')
 
@@ -115,9 +117,9 @@ def test_random_broadcast_patterns(seed):
     assert r.returncode == 0, f'{case}\nrc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
 
 
-@pytest.mark.parametrize('seed', range(100, 106))
+@pytest.mark.parametrize('seed', cases.FUZZ_SEEDS)
 def test_random_recurrences(seed):
     """Random step functions (tests/cases.py: random_step) through the emitted kernels."""
-    dims = ['2,8,2,8,16', '1,19,2,5,32', '2,16,1,24,128', '2,8,2,8,24', '1,19,2,5,48', '2,16,1,12,5'][seed % 6]
+    dims = ','.join(str(d) for d in cases.FUZZ_DIMS[seed % 6])
     r = subprocess.run([sys.executable, RUNNER, f'gen:{seed}', dims, 'f32', str(seed % 2), '1e-4'], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2500:]}\n{r.stderr[-3000:]}'

@@ -67,6 +67,10 @@ def warm(force=False, seen=None):
         step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
         n += len(compile_plan(plan, force=force, seen=seen))
+    for seed in cases.FUZZ_SEEDS:                       # tests/test_gpu_fuzz.py
+        step, xs, ss = cases.fuzz_case(seed, (th.float32, th.bfloat16)[(seed // 6) % 2])
+        plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
+        n += len(compile_plan(plan, force=force, seen=seen))
     for name, dims in GOLDEN.items():
         n += len(compile_plan(prebuild.plan_for(name, dims, th.float32), force=force, seen=seen))
     for name in ('rwkv7', 'gated_delta_rule'):
