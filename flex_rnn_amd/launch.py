@@ -203,6 +203,9 @@ class CompiledPlan:
             return kern
 
         self._load = load
+        self.builds, self.build_times, self._grid, self._packer = {}, {}, {}, {}
+        if plan.B == 0 or plan.T == 0:
+            return                          # nothing will ever be launched for an empty batch or no timesteps
         # Every kernel comes in a few candidate builds (tiles of the row kernels; prefetch depth and
         # occupancy request of the gradient kernel), first-ranked first.  All are loaded; the first
         # call that runs a kernel times its candidates on that call's tensors and keeps the fastest.
@@ -331,6 +334,10 @@ class CompiledPlan:
             tensors[f'sck{k}'] = sck[k]
         for k in range(p.noutputs):
             tensors[f'out{k}'] = outs[k]
+        if B == 0 or T == 0:                       # nothing to scan: the state passes through
+            for a, b in zip(stT, state0):
+                a.copy_(b)
+            return (*outs, *stT, *sck, aux)
         self._tune('frnn_fw', tensors)
         self._launch('frnn_fw', tensors)
         return (*outs, *stT, *sck, aux)
@@ -338,7 +345,7 @@ class CompiledPlan:
     def forward_only(self, inputs: Sequence[th.Tensor], state0: Sequence[th.Tensor]):
         """Outputs and final states only (inference): a forward kernel that writes no checkpoints and
         no saved row sums, built on first use."""
-        if 'frnn_fwi' not in self.kernels:
+        if 'frnn_fwi' not in self.kernels and self.plan.B and self.plan.T:
             self._add_builds('frnn_fwi', [(s_, p_, None) for s_, p_ in row_kernel_builds(self.plan, False, save=False)])
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
@@ -352,6 +359,10 @@ class CompiledPlan:
             tensors[f'stT{k}'] = stT[k]
         for k in range(p.noutputs):
             tensors[f'out{k}'] = outs[k]
+        if pl.B == 0 or pl.T == 0:
+            for a, b in zip(stT, state0):
+                a.copy_(b)
+            return (*outs, *stT)
         self._tune('frnn_fwi', tensors)
         self._launch('frnn_fwi', tensors)
         return (*outs, *stT)
@@ -362,6 +373,12 @@ class CompiledPlan:
         dev = inputs[0].device
         B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.NP          # (hidden buffers have the padded width)
         atomic = set(pl.atomic)
+        if B == 0 or T == 0:                       # no timestep touched any input; d state passes through
+            like = self.state_meta if self.state_meta is not None else [(s.shape, s.stride(), s.dtype) for s in dstateT]
+            dst0 = tuple(th.empty_strided(sh, st, dtype=dt, device=dev) for sh, st, dt in like)
+            for a, b in zip(dst0, dstateT):
+                a.copy_(b)
+            return tuple(th.zeros_like(x) for x in inputs), dst0
         daux = th.empty(len(p.daux), B, H, T, M, dtype=th.float32, device=dev)
         dck = tuple(th.empty(B, H, pl.nchunks, M, N, dtype=th.float32, device=dev) for _ in state_store) \
             if 'frnn_bw2' in self.kernels else ()

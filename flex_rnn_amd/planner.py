@@ -123,6 +123,10 @@ class Plan:
 def classify(inputs, state):
     """Shape validation and operand classes (twopass.py:45-72)."""
     B, T, H = [max(i.shape[j] for i in inputs) for j in range(3)]
+    if state and state[0].ndim == 4 and 0 in (state[0].shape[0], min(i.shape[1] for i in inputs)):
+        # an empty batch or no timesteps: a size of 1 is a broadcast input there, not the extent
+        B = state[0].shape[0]
+        T = 0 if min(i.shape[1] for i in inputs) == 0 else T
     M = max(i.shape[-2] for i in tuple(inputs) + tuple(state))
     N = max(i.shape[-1] for i in tuple(inputs) + tuple(state))
     dims = [B, T, H, M, N]
@@ -271,8 +275,9 @@ def part_input_classes(part: Partition) -> List[str]:
 def make_plan(step: Callable, inputs, state, tile: Optional[TileConfig] = None) -> Tuple[Plan, tuple, tuple]:
     (B, T, H, M, N), cls, bcast = classify(inputs, state)
 
-    inputs_t = [i[:, 0] for i in inputs]
-    res = step(*[i.to('meta') for i in [*inputs_t, *state]])
+    # one timestep's worth of every input, as shapes only (so that T == 0 plans too)
+    inputs_t = [th.empty((i.shape[0], *i.shape[2:]), dtype=i.dtype, device='meta') for i in inputs]
+    res = step(*inputs_t, *[s.to('meta') for s in state])
     output_t, nstate = [r if isinstance(r, tuple) else (r,) for r in res]
     ninputs, noutputs, nstates = len(inputs_t), len(output_t), len(nstate)
     assert len(nstate) == len(state), 'step must return as many states as it takes'

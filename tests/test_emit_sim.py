@@ -123,3 +123,27 @@ def test_random_recurrences(seed):
     dims = ','.join(str(d) for d in cases.FUZZ_DIMS[seed % 6])
     r = subprocess.run([sys.executable, RUNNER, f'gen:{seed}', dims, 'f32', str(seed % 2), '1e-4'], capture_output=True, text=True, timeout=900)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2500:]}\n{r.stderr[-3000:]}'
+
+
+@pytest.mark.parametrize('dims', [(0, 16, 2, 16, 16), (2, 0, 2, 16, 16)])
+def test_empty_batch_and_empty_time(dims):
+    """No batch entries or no timesteps: nothing is launched, the state and its gradient pass
+    through, outputs and per-step gradients are empty, gradients of broadcast inputs zero."""
+    import torch as th
+    from flex_rnn_amd import planner
+    from hipsim import SimPlan
+    step, xs, ss = cases.make_inputs('mamba', *dims, dtype=th.float32)
+    ss = [th.randn(s.shape) for s in ss]
+    plan, fm, bm = planner.make_plan(step, xs, ss)
+    nout, nst = plan.part.noutputs, plan.part.nstates
+    sp = SimPlan(plan, state_meta=fm[nout:nout + nst])
+    res = sp.forward(tuple(xs), tuple(ss))
+    outs, stT, sck, aux = res[:nout], res[nout:nout + nst], res[nout + nst:nout + 2 * nst], res[-1]
+    assert [tuple(r.shape) for r in res] == [tuple(sh) for sh, _, _ in fm]
+    assert all(th.equal(a, b) for a, b in zip(stT, ss)) and all(o.numel() == 0 for o in outs)
+    lean = sp.forward_only(tuple(xs), tuple(ss))
+    assert all(th.equal(a, b) for a, b in zip(lean[nout:], ss))
+    dS = [th.randn(s.shape) for s in ss]
+    dins, dst0 = sp.backward(tuple(th.zeros_like(o) for o in outs), tuple(dS), tuple(xs), sck, aux)
+    assert all(th.equal(a, b) for a, b in zip(dst0, dS))
+    assert all(d.shape == x.shape and not d.any() for d, x in zip(dins, xs))

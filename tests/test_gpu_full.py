@@ -341,3 +341,21 @@ def test_hip_graph_capture_and_replay():
         th.cuda.synchronize()
         for a, b in zip(got, want):          # equal up to the order of fp32 atomic additions
             assert recurrence.rel_err(a, b) < 5e-3, it
+
+
+@pytest.mark.parametrize('dims', [(0, 16, 2, 16, 16), (2, 0, 2, 16, 16)])
+def test_empty_batch_and_empty_time(dims):
+    """Nothing to scan: outputs are empty, the state passes through, and so does its gradient."""
+    print(f'case empty {dims}', flush=True)
+    step, xs, ss = cases.make_inputs('mamba', *dims, dtype=th.float32)
+    xg = [x.cuda().requires_grad_() for x in xs]
+    sg = [th.randn(s.shape).cuda().requires_grad_() for s in ss]
+    f = flex_rnn_amd.jit(step, n_step_args=len(xs) + len(ss))
+    y, S = f(*xg, *sg)
+    assert y.shape == (dims[0], dims[1], dims[2], dims[3]) and th.equal(S, sg[0])
+    dS = th.randn_like(S)
+    grads = th.autograd.grad([y, S], xg + sg, [th.zeros_like(y), dS])
+    assert th.equal(grads[-1], dS)
+    assert all(g.shape == x.shape and not g.any() for g, x in zip(grads, xg))
+    y2, S2 = f.infer(*xg, *sg)
+    assert y2.shape == y.shape and th.equal(S2, sg[0])
