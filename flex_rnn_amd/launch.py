@@ -14,6 +14,7 @@ import contextlib
 import dataclasses
 import os
 import struct
+import threading
 from concurrent.futures import ThreadPoolExecutor
 from typing import Dict, List, Sequence, Tuple
 
@@ -33,6 +34,7 @@ def kernel_specs(plan, prefetch: int = 4) -> List[KernelSpec]:
     return [em.fw(), em.bw1()] + ([em.bw2(prefetch=prefetch)] if needs_gradient_kernel(plan.part) else [])
 
 
+_seen_lock = threading.Lock()
 MAX_SPILL_BYTES = 64      # per lane; the untimed choice among gradient-kernel builds does not accept more
 
 
@@ -40,9 +42,10 @@ def _compile(specs, force, seen):
     jobs = []
     for s in specs:
         key = runtime.source_key(s.name, s.source)
-        again = force and (seen is None or key not in seen)
-        if seen is not None:
-            seen.add(key)
+        with _seen_lock:                    # (plans are compiled from several threads at warm-up)
+            again = force and (seen is None or key not in seen)
+            if seen is not None:
+                seen.add(key)
         jobs.append((s, again))
     # independent compiler processes: wait for them side by side (the runtime call releases the GIL)
     def one(j):
@@ -172,6 +175,14 @@ def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec,
         spec, path, _ = gradient_kernel_builds(plan, force, seen)[0]
         built.append((spec, path))
     return built
+
+
+def compile_plans(plans, force: bool = False, seen=None, workers: int = 3) -> int:
+    """`compile_plan` for several plans, `workers` of them side by side (a plan's own compiler runs
+    do not keep all cores busy: its gradient kernel takes much longer than the rest).  Returns the
+    number of kernels `compile_plan` handed back."""
+    with ThreadPoolExecutor(max_workers=max(1, workers)) as pool:
+        return sum(len(b) for b in pool.map(lambda pl: compile_plan(pl, force=force, seen=seen), plans))
 
 
 class CompiledPlan:

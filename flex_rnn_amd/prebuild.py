@@ -7,6 +7,7 @@ cache.  `CASES` lists the workloads the test-suite, the smoke test and the bench
 """
 from __future__ import annotations
 
+from concurrent.futures import ThreadPoolExecutor
 from typing import Iterable, List, Optional, Tuple
 
 import torch as th
@@ -60,12 +61,15 @@ def _is_full(name: str, i: int, j: int) -> bool:
 
 
 def warm(cases: Iterable = CASES, verbose: bool = False, force: bool = False) -> int:
-    n = 0
+    cases = list(cases)
+    plans = [plan_for(name, dims, dtype) for name, dims, dtype in cases]       # (tracing: one at a time)
     seen = set()
-    for name, dims, dtype in cases:
-        plan = plan_for(name, dims, dtype)
-        for spec, path in compile_plan(plan, force=force, seen=seen):
-            n += 1
-            if verbose:
-                print(f'  {name} {dims or "full"} {spec.name}: {path}')
+    n = 0
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        built = pool.map(lambda pl: compile_plan(pl, force=force, seen=seen), plans)
+        for (name, dims, dtype), specs in zip(cases, built):
+            for spec, path in specs:
+                n += 1
+                if verbose:
+                    print(f'  {name} {dims or "full"} {spec.name}: {path}')
     return n

@@ -12,6 +12,7 @@ import json
 import os
 import re
 import subprocess
+import threading
 from typing import Sequence
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
@@ -146,7 +147,7 @@ def _record_resources(hsaco: str) -> None:
         if m:
             vals[k] = int(m.group(1))
     if len(vals) == len(_RES_FIELDS):
-        tmp = f'{base}.res.tmp{os.getpid()}'
+        tmp = f'{base}.res.tmp{os.getpid()}_{threading.get_ident()}'      # (threads of one process compile side by side)
         with open(tmp, 'w') as f:
             json.dump(vals, f)
         os.replace(tmp, base + '.res')

@@ -39,6 +39,18 @@ def test_compile_cache_hit_and_miss(runtime_lib, tmp_path, monkeypatch):
     assert os.path.getsize(p1) > 0
 
 
+def test_threads_compiling_the_same_key(runtime_lib, tmp_path, monkeypatch):
+    """Warm-up compiles plans from several threads, and plans share kernels: the compiler runs once,
+    every thread gets the same path, and no temporary file of one thread is taken by another."""
+    from concurrent.futures import ThreadPoolExecutor
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    src = TRIVIAL + '// threads\n'
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        paths = list(pool.map(lambda _: runtime.compile_kernel('k', src), range(4)))
+    assert len(set(paths)) == 1 and os.path.getsize(paths[0]) > 0
+    assert not [f for f in os.listdir(tmp_path) if '.tmp' in f]
+
+
 def test_compile_error_is_reported(runtime_lib, tmp_path, monkeypatch):
     monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
     with pytest.raises(RuntimeError, match='hipcc failed'):

@@ -11,7 +11,7 @@ if HERE not in sys.path:
 
 import cases  # noqa: E402
 from flex_rnn_amd import configs, planner, prebuild  # noqa: E402
-from flex_rnn_amd.launch import compile_plan  # noqa: E402
+from flex_rnn_amd.launch import compile_plans  # noqa: E402
 
 OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn', (2, 32, 2, 32, 16)),
          ('hgrn', (2, 64, 1, 256, 1)), ('rwkv4', (2, 32, 1, 64, 1)), ('mlstm_gates', (2, 32, 2, 32, 1)),
@@ -26,20 +26,17 @@ OTHER = [('rwkv6', (2, 32, 2, 32, 32)), ('s4d', (2, 32, 1, 16, 32)), ('longhorn'
 EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
 
 
-def warm_examples(force=False, seen=None):
-    """Dry-runs every example layer on meta tensors, captures the plans its jit objects
-    request and compiles their kernels."""
+def example_plans():
+    """Dry-runs every example layer on meta tensors and returns the plans its jit objects request."""
     import flex_rnn_amd
     jit_mod = sys.modules['flex_rnn_amd.jit']        # (the package attribute `jit` is the class)
     from flex_rnn_amd import examples
-    n = 0
+    plans = []
     orig = jit_mod.build_twopass
 
     def capture(step, inputs, state, dryrun=False, tile=None):
-        nonlocal n
         metas = [t.to('meta') for t in inputs], [t.to('meta') for t in state]
-        plan = planner.make_plan(step, *metas, tile)[0]
-        n += len(compile_plan(plan, force=force, seen=seen))
+        plans.append(planner.make_plan(step, *metas, tile)[0])
         return orig(step, inputs, state, dryrun=True, tile=tile)
 
     jit_mod.build_twopass = capture
@@ -50,7 +47,7 @@ def warm_examples(force=False, seen=None):
             layer(*inputs)
     finally:
         jit_mod.build_twopass = orig
-    return n
+    return plans
 
 
 GOLDEN = {'delta_rule': (1, 6, 2, 4, 4), 'mamba1': (2, 6, 2, 4, 4), 'mamba2': (2, 6, 2, 4, 8),
@@ -58,30 +55,30 @@ GOLDEN = {'delta_rule': (1, 6, 2, 4, 4), 'mamba1': (2, 6, 2, 4, 4), 'mamba2': (2
 
 
 def warm(force=False, seen=None):
-    n = warm_examples(force, seen)
+    plans = example_plans()
     for name, dims in OTHER:
         step, xs, ss = cases.make_inputs(name, *dims, dtype=th.float32)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
-        n += len(compile_plan(plan, force=force, seen=seen))
+        plans.append(plan)
     for dtype in (th.float16, th.float64):
         step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
-        n += len(compile_plan(plan, force=force, seen=seen))
+        plans.append(plan)
     for seed in cases.FUZZ_SEEDS:                       # tests/test_gpu_fuzz.py
         step, xs, ss = cases.fuzz_case(seed, (th.float32, th.bfloat16)[(seed // 6) % 2])
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
-        n += len(compile_plan(plan, force=force, seen=seen))
+        plans.append(plan)
     for name, dims in GOLDEN.items():
-        n += len(compile_plan(prebuild.plan_for(name, dims, th.float32), force=force, seen=seen))
+        plans.append(prebuild.plan_for(name, dims, th.float32))
     for name in ('rwkv7', 'gated_delta_rule'):
         B, T, H, M, N = configs.DEFAULT_DIMS[name]
-        n += len(compile_plan(prebuild.plan_for(name, (B, 128, H, M, N)), force=force, seen=seen))
-    n += len(compile_plan(prebuild.plan_for('rwkv7', (8, 512, 32, 128, 128)), force=force, seen=seen))
-    n += len(compile_plan(prebuild.plan_for('mamba2', (2, 64, 4, 64, 128)), force=force, seen=seen))
+        plans.append(prebuild.plan_for(name, (B, 128, H, M, N)))
+    plans.append(prebuild.plan_for('rwkv7', (8, 512, 32, 128, 128)))
+    plans.append(prebuild.plan_for('mamba2', (2, 64, 4, 64, 128)))
     for name in ('rwkv7', 'mamba1', 'mamba2'):
         B, T, H, M, N = configs.DEFAULT_DIMS[name]
-        n += len(compile_plan(prebuild.plan_for(name, (2, 77, 2, M, N)), force=force, seen=seen))
+        plans.append(prebuild.plan_for(name, (2, 77, 2, M, N)))
     for name, dims in [('rwkv7', (2, 77, 2, 128, 128)), ('mamba1', (2, 45, 4, 128, 16)),
                        ('gated_delta_rule', (2, 1, 2, 128, 128)), ('mamba2', (2, 19, 4, 64, 128))]:
-        n += len(compile_plan(prebuild.plan_for(name, dims, th.float32), force=force, seen=seen))
-    return n
+        plans.append(prebuild.plan_for(name, dims, th.float32))
+    return compile_plans(plans, force=force, seen=seen)
