@@ -114,6 +114,10 @@ def main():
         per.setdefault(kname, []).append(e0.elapsed_time(e1))
     kavg = {k: sum(v) / len(v) for k, v in per.items()}
     dominant = max(kavg, key=kavg.get)
+    # per step: the kernels' durations added up; median and 20 / 80 % quantiles over the timed steps
+    per_step = sorted(sum(v[i] for v in per.values()) for i in range(min(len(v) for v in per.values())))
+    quantiles = {q: round(per_step[min(len(per_step) - 1, int(p * len(per_step)))], 4)
+                 for q, p in (('p20', 0.2), ('median', 0.5), ('p80', 0.8))}
     w = WORK[name]
     elems = B * T * H * M * N
     kflop = {'frnn_fw': w['flop_fwd'], 'frnn_bw1': w['flop_bwd'] - w['flop_bw2'], 'frnn_bw2': w['flop_bw2']}
@@ -169,6 +173,7 @@ def main():
         'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
         'roofline': roofline, 'cpu_baseline': cpu,
         'gpu_kernel_ms_per_step': round(gpu_ms, 4),
+        'gpu_kernel_ms_per_step_quantiles': quantiles,
         # candidate builds of the gradient kernel as timed on the first backward call (the fastest runs)
         'row_kernel_builds': {k: {'tiles (L, C, R, W)': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
                                   'ms': compiled.build_times.get(k) and [round(v, 4) for v in compiled.build_times[k]]}
