@@ -749,6 +749,17 @@ class Emitter:
                         f'  for (int c = 0; c < {C}; c++) gmacc{i}[r][c] = 0.0f;\n')
         body.append(f'  const int tlast = ((T - 1) / {TS}) * {TS};\n')
         body.append(stg.load('tlast', '  '))
+
+        def ckpt_fetch(k, chunk, indent):
+            """The state checkpoint of `chunk` into the registers pS<k>: issued one chunk ahead, like the
+            staged operands, so that no chunk starts by waiting for HBM."""
+            rr, cc = _dims(st_ext[k], R, C)
+            return (f'#pragma unroll\n{indent}for (int r = 0; r < {rr}; r++)\n#pragma unroll\n{indent}for (int c = 0; c < {cc}; c++) '
+                    f'pS{k}[r][c] = ((const float*){A.p(f"sck{k}")})[(((i64)(b * H + h) * nch + ({chunk})) * M + ROWC(r)) * {self.NP} + COL(c)];\n')
+
+        for k in range(nst if needs_state else 0):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'  float pS{k}[{rr}][{cc}];\n' + ckpt_fetch(k, f'tlast / {DT}', '  '))
         body.append(f'  for (int t0 = tlast; t0 >= 0; t0 -= {TS}) {{\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
         # d_state checkpoints are only read by the gradient kernel
@@ -761,7 +772,12 @@ class Emitter:
         body.append('    }\n    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
-        body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ') + '    }\n')
+        for k in range(nst if needs_state else 0):
+            rr, cc = _dims(st_ext[k], R, C)
+            body.append(f'    float Sh{k}_0[{rr}][{cc}];\n#pragma unroll\n    for (int r = 0; r < {rr}; r++)\n'
+                        f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = pS{k}[r][c];\n')
+        body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ')
+                    + ''.join(ckpt_fetch(k, f't0 / {DT} - 1', '      ') for k in range(nst if needs_state else 0)) + '    }\n')
 
         # With state recompute a timestep's operands are read by `bw_restep` and again by
         # `bw_dstep`.  Those without a column extent (one register per row) are loaded once for
@@ -844,11 +860,6 @@ class Emitter:
             body.append('    }\n')
         else:
             # recompute the DT states of this chunk from its checkpoint, then walk back
-            for k in range(nst):
-                rr, cc = _dims(st_ext[k], R, C)
-                body.append(f'    float Sh{k}_0[{rr}][{cc}];\n#pragma unroll\n    for (int r = 0; r < {rr}; r++)\n'
-                            f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = '
-                            f'((const float*){A.p(f"sck{k}")})[(((i64)(b * H + h) * nch + (t0 / {DT})) * M + ROWC(r)) * {self.NP} + COL(c)];\n')
             for tt in range(1, DT):
                 for k in range(nst):
                     rr, cc = _dims(st_ext[k], R, C)
