@@ -202,6 +202,12 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     while C > 2 and N // (C // 2) <= 64 and waves < 2 * 4 * n_cu:
         C //= 2
         L, G, R, W, waves = geometry(C)
+    if part.dstep_needs_state:
+        # several states there leave chunks of under 8 steps at 8 columns per lane, and the forward kernel then
+        # spends its time storing checkpoints (S4D, two states: 1.05 -> 0.64 ms with 4 columns per lane)
+        while C > 2 and N // (C // 2) <= 64 and 64 // (C * part.nstates) < 8:
+            C //= 2
+            L, G, R, W, waves = geometry(C)
     MT = W * G * R
     R1 = W1 = 0
     if part.dstep_needs_state:
