@@ -111,6 +111,8 @@ __device__ __forceinline__ void atomic_addf(void* p, i64 i, float v) {
   __hip_atomic_fetch_add(((float*)p) + i, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float f_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// a value that is the same on every lane of the wave, moved to a scalar register
+__device__ __forceinline__ float wave_uniform(float x) { return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x))); }
 __device__ __forceinline__ float f_sigmoid(float x) { return 1.0f / (1.0f + __expf(-x)); }
 __device__ __forceinline__ float f_tanh(float x) { return 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f); }
 __device__ __forceinline__ float f_sign(float x) { return x > 0.0f ? 1.0f : (x < 0.0f ? -1.0f : 0.0f); }
@@ -1108,6 +1110,7 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         for j in loop_ops:
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
+        n_uniform = sum(1 for f in rfront if self.jext[f] == (False, False))
         if rfront:
             for tt in range(DT):
                 call = []
@@ -1121,6 +1124,14 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
                     b.append(f'  float g{q}_{tt}[1][1];\n')
                     call.append(f'g{q}_{tt}')
                 b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
+                # With one instance per wave a value without row and column extent is the same on all lanes;
+                # kept in a scalar register it costs no vector register for the length of the chunk (Mamba-2's
+                # per-step decay: 184 -> 150 registers, three waves per SIMD without spills).  The scalar
+                # inputs themselves stay in vector registers: as scalar operands of the row loop's
+                # multiply-adds they cost moves (gated delta rule: 7 % slower).
+                for q, f in enumerate(rfront):
+                    if IPB == 1 and self.jext[f] == (False, False) and n_uniform * DT <= 32:      # (more would spill scalar registers)
+                        b.append(f'  g{q}_{tt}[0][0] = wave_uniform(g{q}_{tt}[0][0]);\n')
         # ---- per-row operands of the chunk go through LDS: staged once per row block by the
         # instance's own lanes (coalesced along m), read back per row as broadcast vectors
         rowops = []          # (lds name, loader(tt, mexpr) -> expr, register prefix)

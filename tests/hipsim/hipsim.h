@@ -122,6 +122,8 @@ static inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int ro
   return sim_lane_read(src, s);
 }
 
+static inline int __builtin_amdgcn_readfirstlane(int v) { return sim_lane_read(v, 0); }
+
 static inline float __shfl_xor(float v, int mask, int width = 64) {
   (void)width;
   int i;
