@@ -126,8 +126,11 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
 def row_kernel_tiles(plan, reverse: bool):
     """(L, C, R, W) candidates for the forward kernel (or the reverse scan): the heuristic's choice
     first; half the rows per lane (more, lighter waves) with the same and with twice the waves per
-    workgroup; and, where the heuristic spread a state row over more than one 16-lane DPP row to get
-    more waves, twice the columns per lane (cheaper reductions, fewer waves).  Which is fastest
+    workgroup; where the heuristic spread a state row over more than one 16-lane DPP row to get
+    more waves, twice the columns per lane (cheaper reductions, fewer waves); and, for a state row of
+    one DPP row, twice the columns and half the rows per lane with twice the waves per workgroup (the
+    same state registers per lane, one reduction step fewer shared by twice the columns, and a
+    workgroup that stages the row operands of twice the rows).  Which is fastest
     depends on how many (batch, head) pairs there are, on the LDS traffic of the staged operands
     and on register use; the first call times them."""
     t = plan.tile
@@ -149,6 +152,8 @@ def row_kernel_tiles(plan, reverse: bool):
     if t.L > 16 and t.C < 8:
         add(t.L // 2, t.C * 2, R, W)
         add(t.L // 2, t.C * 2, R, 2 * W)
+    if t.L == 16 and t.C == 8 and R > 1 and not fixed_r:
+        add(8, 16, R // 2, 2 * W)
     return out
 
 
