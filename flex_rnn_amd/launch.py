@@ -302,31 +302,36 @@ class CompiledPlan:
 
     def _tune(self, name, tensors, accumulators=()):
         """Times every candidate build of kernel `name` on the tensors of this call (one untimed
-        run, then the faster of two timed ones) and keeps the fastest.  The kernels only store and
+        run, then the fastest of three timed ones, in rounds over the candidates) and keeps the
+        fastest.  The kernels only store and
         accumulate; `accumulators` (what they add into) are put back afterwards.  Synchronises,
         once per kernel and plan; skipped while the stream is being captured."""
         if name not in self._tune_pending or th.cuda.is_current_stream_capturing():
             return
         self._tune_pending.discard(name)
         saved = [a.clone() for a in accumulators]
-        times = []
-        for i in range(len(self.builds[name])):
-            self._select(name, i)
-            best = float('inf')
-            try:
-                self._launch(name, tensors)
-                for _ in range(2):
+        n = len(self.builds[name])
+        times = [float('inf')] * n
+        usable = [True] * n
+        # rounds over all candidates (the first untimed) rather than one candidate after the other: the
+        # clock ramps up over the first launches, and whoever ran first would be timed on a cold chip
+        for rnd in range(4):
+            for i in range(n):
+                if not usable[i]:
+                    continue
+                self._select(name, i)
+                try:
                     e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
                     e0.record()
                     self._launch(name, tensors)
                     e1.record()
                     e1.synchronize()
-                    best = min(best, e0.elapsed_time(e1))
-            except runtime.RuntimeError_:
-                if i == 0:
-                    raise                       # the first-ranked build must be launchable
-                best = float('inf')             # (a candidate the device refuses to launch is just not taken)
-            times.append(best)
+                    if rnd:
+                        times[i] = min(times[i], e0.elapsed_time(e1))
+                except runtime.RuntimeError_:
+                    if i == 0:
+                        raise                   # the first-ranked build must be launchable
+                    usable[i] = False           # (a candidate the device refuses to launch is just not taken)
         self._select(name, min(range(len(times)), key=times.__getitem__))
         self.build_times[name] = times
         for a, s_ in zip(accumulators, saved):
