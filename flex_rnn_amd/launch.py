@@ -190,6 +190,14 @@ def compile_plans(plans, force: bool = False, seen=None, workers: int = 3) -> in
         return sum(len(b) for b in pool.map(lambda pl: compile_plan(pl, force=force, seen=seen), plans))
 
 
+def _fixed_picks() -> Dict[str, int]:
+    """`FLEX_RNN_PICK="frnn_fw=3,frnn_bw1=3"`: the candidate build to run for the named kernels, by its
+    position in the candidate list, instead of timing them (profiles of one build per kernel;
+    repeatable runs).  Kernels not named are timed as usual."""
+    spec = os.environ.get('FLEX_RNN_PICK', '')
+    return {k.strip(): int(v) for k, v in (kv.split('=') for kv in spec.split(',') if kv.strip())}
+
+
 class CompiledPlan:
     _tune_pending = frozenset()
 
@@ -236,10 +244,11 @@ class CompiledPlan:
             self.builds = {k: [(s_, load(s_, p_), r_) for s_, p_, r_ in v] for k, v in built.items()}
         self.build_times = {}
         tune = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
-        self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1}
+        picks = _fixed_picks()
+        self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1 and k not in picks}
         self._grid, self._packer = {}, {}
         for k, v in self.builds.items():
-            self._select(k, 0)
+            self._select(k, picks.get(k, 0))
 
     @property
     def bw2_builds(self):
@@ -250,6 +259,8 @@ class CompiledPlan:
         return self.build_times.get('frnn_bw2')
 
     def _select(self, name, index):
+        assert 0 <= index < len(self.builds[name]), \
+            f'{name} has {len(self.builds[name])} candidate builds, number {index} was asked for'
         spec, kern, _ = self.builds[name][index]
         self.kernels[name] = (spec, kern)
         self._register(name, spec)
@@ -264,9 +275,10 @@ class CompiledPlan:
         on_gpu = self.device is not None and self.device.type == 'cuda'
         with (th.cuda.device(self.device) if on_gpu else contextlib.nullcontext()):
             self.builds[name] = [(s_, self._load(s_, p_), r_) for s_, p_, r_ in built]
-        if len(built) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0':
+        picks = _fixed_picks()
+        if len(built) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0' and name not in picks:
             self._tune_pending.add(name)
-        self._select(name, 0)
+        self._select(name, picks.get(name, 0))
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):

@@ -170,3 +170,11 @@ def test_dynamo_traces_through_the_op_without_graph_break(runtime_lib):
     assert len(graphs) == 1
     targets = [str(n.target) for n in graphs[0].graph.nodes if n.op == 'call_function']
     assert sum('flex_rnn.fw_' in t for t in targets) == 1, targets
+
+
+def test_fixed_pick_switch_is_parsed(monkeypatch):
+    from flex_rnn_amd import launch
+    monkeypatch.delenv('FLEX_RNN_PICK', raising=False)
+    assert launch._fixed_picks() == {}
+    monkeypatch.setenv('FLEX_RNN_PICK', 'frnn_fw=3, frnn_bw1=1')
+    assert launch._fixed_picks() == {'frnn_fw': 3, 'frnn_bw1': 1}
