@@ -178,3 +178,21 @@ def test_fixed_pick_switch_is_parsed(monkeypatch):
     assert launch._fixed_picks() == {}
     monkeypatch.setenv('FLEX_RNN_PICK', 'frnn_fw=3, frnn_bw1=1')
     assert launch._fixed_picks() == {'frnn_fw': 3, 'frnn_bw1': 1}
+
+
+def test_row_kernel_candidate_tiles_are_valid():
+    """Every candidate tile of the row kernels covers the state row, keeps the workgroup within the
+    state's rows and passes the planner's own check; the headline shape offers the wide-column tile."""
+    import dataclasses
+    from flex_rnn_amd import launch, planner, prebuild
+    for name in ('rwkv7', 'mamba2', 'gated_delta_rule', 'mamba1'):
+        plan = prebuild.plan_for(name)
+        for reverse in (False, True):
+            tiles = launch.row_kernel_tiles(plan, reverse)
+            assert tiles[0][:2] == (plan.tile.L, plan.tile.C) and len(set(tiles)) == len(tiles) <= 5
+            for L, C, r, w in tiles:
+                assert L * C == plan.NP and (64 // L) * r * w <= max(plan.M, (64 // L) * r)
+                t = dataclasses.replace(plan.tile, L=L, C=C)
+                t = dataclasses.replace(t, R1=r, W1=w) if reverse else dataclasses.replace(t, R=r, W=w)
+                planner.check_tile(t, plan.H, plan.NP, plan.part)
+    assert (8, 16, 2, 8) in launch.row_kernel_tiles(prebuild.plan_for('rwkv7'), False)
