@@ -76,6 +76,9 @@ TILED = [
     ('cfg:rwkv7', '1,16,1,128,128', 'f32', 0, 'R=2,W=8,R1=2,W1=4'),
     ('cfg:mamba2', '1,16,2,64,128', 'f32', 1, 'R=1,W=8,R1=1,W1=8'),
     ('cfg:mamba1', '2,16,2,128,16', 'f32', 0, 'R=1,W=8,R1=1,W1=8'),
+    # 16 columns per lane (a state row of 128 in 8 lanes: three reduction steps), one workgroup per head
+    ('cfg:rwkv7', '1,19,2,128,128', 'bf16', 1, 'L=8,C=16,R=2,W=8,R1=2,W1=8'),
+    ('cfg:mamba2', '1,16,2,64,128', 'f32', 0, 'L=8,C=16,R=1,W=8,R1=1,W1=8'),
 ]
 
 
