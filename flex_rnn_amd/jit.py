@@ -39,7 +39,7 @@ class jit:
         self.forward_func = self.backward_func = None
         self.is_dynamic = bool(dynamic)
         self._entries = {}        # dynamic mode: argument signature -> plan entry
-        self._bw_index = {}       # dynamic mode: (input signature, checkpoint shapes) -> plan entry
+        self._by_id = {}          # dynamic mode: entry number -> plan entry (see `_tag`)
         if n_step_args is None:
             n_step_args = len(inspect.signature(step).parameters)
         # arity: run the step once on 1x1 meta tensors (jit.py:13-16)
@@ -65,17 +65,26 @@ class jit:
                 e['fw_meta'], e['bw_meta'] = build_twopass(self.step, inputs, state, dryrun=True)
         elif 'forward' not in e:
             e['forward'], e['backward'], e['fw_meta'], e['bw_meta'] = build_twopass(self.step, inputs, state)
-        nout, nst = self.noutputs, self.nstates
-        stores = tuple(tuple(sh) for sh, _, _ in e['fw_meta'][nout + nst:nout + 2 * nst])
-        self._bw_index[_sig(inputs) + stores] = e
+        if 'id' not in e:
+            e['id'] = len(self._by_id) + 1
+            self._by_id[e['id']] = e
         self.fw_meta, self.bw_meta = e['fw_meta'], e['bw_meta']
         self.forward_func, self.backward_func = e.get('forward'), e.get('backward')
         return e
 
-    def _bw_entry(self, inputs, state_store):
-        key = _sig(inputs) + tuple(tuple(int(n) for n in s.shape) for s in state_store)
-        assert key in self._bw_index, 'backward called with tensors no forward call has produced'
-        return self._bw_index[key]
+    @staticmethod
+    def _tag(e, device):
+        """Dynamic mode: a hidden result without elements whose *shape* `[0, entry number]` names the plan
+        entry of a forward call.  It is saved for backward with the checkpoints, so the backward operator
+        finds the plan of exactly that forward call from static metadata alone (it also survives
+        tracing by `torch.compile`): two signatures that differ only in the state's dtype or strides
+        have the same inputs and checkpoint shapes and could not be told apart by those."""
+        return th.empty((0, e['id']), dtype=th.uint8, device=device)
+
+    def _bw_entry(self, tag):
+        assert tag.ndim == 2 and tag.shape[0] == 0 and tag.shape[1] in self._by_id, \
+            'backward called with tensors no forward call has produced'
+        return self._by_id[tag.shape[1]]
 
     def infer(self, *args):
         """Outputs and final states without the ability to differentiate: the forward kernel then
@@ -123,6 +132,7 @@ class jit:
         uid = uuid.uuid4().hex
         nin, nst, nout = self.ninputs, self.nstates, self.noutputs
         naux = 1        # all saved row-sums travel in one packed tensor (jit.py:43)
+        ntag = 1 if self.is_dynamic else 0      # dynamic mode: one more hidden result, see `_tag`
 
         def metas(meta, device):
             return tuple(th.empty_strided(shape, stride, dtype=dtype, device=device) for shape, stride, dtype in meta)
@@ -136,7 +146,7 @@ class jit:
             return hit[1]
 
         fw_schema = '(' + ', '.join(f'Tensor x{i}' for i in range(nin + nst)) + ') -> (' \
-            + ', '.join(['Tensor'] * (nout + 2 * nst + naux)) + ')'
+            + ', '.join(['Tensor'] * (nout + 2 * nst + naux + ntag)) + ')'
 
         @th.library.custom_op('flex_rnn::fw_' + uid, mutates_args=(), schema=fw_schema)
         def apply(*args):
@@ -145,7 +155,7 @@ class jit:
                 e = self._entry(inputs, state, dry=False)
                 r = e['forward'](inputs, state)
                 verify_meta(r, expected(e['fw_meta']))
-                return r
+                return (*r, self._tag(e, args[0].device))
             if self.forward_func is None:
                 self.forward_func, self.backward_func, self.fw_meta, self.bw_meta = \
                     build_twopass(self.step, inputs, state)
@@ -157,19 +167,20 @@ class jit:
         def _(*args):
             inputs, state = split_list(args, [nin, nst])
             if self.is_dynamic:
-                return metas(self._entry(inputs, state, dry=True)['fw_meta'], args[0].device)
+                e = self._entry(inputs, state, dry=True)
+                return (*metas(e['fw_meta'], args[0].device), self._tag(e, args[0].device))
             if not hasattr(self, 'fw_meta'):
                 self.fw_meta, self.bw_meta = build_twopass(self.step, inputs, state, dryrun=True)
             return metas(self.fw_meta, args[0].device)
 
-        bw_schema = '(' + ', '.join(f'Tensor x{i}' for i in range(nout + 2 * nst + nin + naux)) + ') -> (' \
+        bw_schema = '(' + ', '.join(f'Tensor x{i}' for i in range(nout + 2 * nst + nin + naux + ntag)) + ') -> (' \
             + ', '.join(['Tensor'] * (nin + nst)) + ')'
 
         @th.library.custom_op('flex_rnn::bw_' + uid, mutates_args=(), schema=bw_schema)
         def backward_inner(*args):
-            doutput, dstateT, inputs, state_store, aux = split_list(args, [nout, nst, nin, nst, naux])
+            doutput, dstateT, inputs, state_store, aux, tag = split_list(args, [nout, nst, nin, nst, naux, ntag])
             if self.is_dynamic:
-                e = self._bw_entry(inputs, state_store)
+                e = self._bw_entry(tag[0])
                 dinputs, dstate0 = e['backward'](doutput, dstateT, inputs, state_store, aux)
                 verify_meta(dinputs + dstate0, expected(e['bw_meta']))
                 return (*dinputs, *dstate0)
@@ -180,8 +191,7 @@ class jit:
         @backward_inner.register_fake
         def _(*args):
             if self.is_dynamic:
-                _, _, inputs, state_store, _ = split_list(args, [nout, nst, nin, nst, naux])
-                return metas(self._bw_entry(inputs, state_store)['bw_meta'], args[0].device)
+                return metas(self._bw_entry(args[-1])['bw_meta'], args[0].device)
             return metas(self.bw_meta, args[0].device)
 
         def setup_context(ctx, inputs, output):

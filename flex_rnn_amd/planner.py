@@ -116,8 +116,14 @@ class Plan:
 
     @property
     def atomic(self) -> List[int]:
+        """Inputs whose gradient is accumulated in fp32 (zero-filled, cast back afterwards): those
+        broadcast over batch, time or heads, the row / scalar inputs of a row-split gradient kernel,
+        and every matrix input.  A matrix input has no time axis, so its gradient is a sum over the
+        timesteps and the kernels always form it in fp32 - also at T == 1, where its size-1 time axis
+        does not count as a broadcast."""
         split = set(self.part.row_idx + self.part.scalar_idx) if self.tile.MS > 1 else set()
-        return [i for i, b in enumerate(self.in_bcast) if any(b) or i in split]
+        mats = set(self.part.mat_idx)
+        return [i for i, b in enumerate(self.in_bcast) if any(b) or i in split or i in mats]
 
 
 def classify(inputs, state):
@@ -345,6 +351,12 @@ def build_twopass(step: Callable, inputs, state, dryrun: bool = False, tile: Opt
         return compiled.forward(tuple(inputs_), tuple(state0))
 
     def backward(doutput, dstateT_, inputs_, state_store_, aux_):
+        # (gradients arrive in whatever layout autograd gives them; the kernels take them contiguous.  Shape and
+        # dtype must be those of the final states this plan produced - twopass.py:346 - or the reverse scan
+        # would read them with the wrong element size.)
+        for k, (g, m) in enumerate(zip(dstateT_, fw_out_meta[nout:nout + nst])):
+            assert g.shape == m.shape and g.dtype == m.dtype, \
+                f'final-state gradient #{k+1}: {tuple(g.shape)} {g.dtype} does not match compilation ({tuple(m.shape)} {m.dtype})'
         doutput, dstateT_ = [tuple(i.contiguous() for i in j) for j in (doutput, dstateT_)]
         verify_meta(inputs_, in_meta)
         verify_meta(doutput, fw_out_meta[:nout])

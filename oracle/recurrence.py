@@ -16,6 +16,16 @@ Pinned by (tests/test_oracle.py):
 Gradients of the oracle are `torch.autograd.grad` through this loop (what
 /root/reference/flex_rnn/check_grad.py:30-35 does), pinned by `torch.autograd.gradcheck`
 in fp64 on tiny shapes.
+
+`rel_err` / `assert_close` are the metric and the assertion of every parity test
+(/root/reference/flex_rnn/check_grad.py:20).  Pinned by known values (3-4-5 triangle, the 1e-30
+floor for a zero reference, promotion of bf16 operands to double, asymmetry in its arguments) and
+by negative tests: a result off by twice the tolerance must fail `assert_close`.
+
+`chunked_loop_with_grads` is `loop_with_grads` with bounded memory for long sequences: the same
+loop and the same autograd, one chunk of timesteps at a time, the gradient of the chunk's entry
+state handed back to the chunk before.  Pinned by equality (fp64, 1e-12) with `loop_with_grads`
+on short sequences, chunk lengths that do not divide T and time-broadcast inputs included.
 """
 from __future__ import annotations
 
@@ -55,6 +65,21 @@ def rel_err(a, b):
     return float((a - b).norm() / max(float(b.norm()), 1e-30))
 
 
+def assert_close(got, want, tol, what=''):
+    """The parity assertion: `rel_err(got, want) < tol` (and equal shapes); returns the error."""
+    assert tuple(got.shape) == tuple(want.shape), f'{what}: shape {tuple(got.shape)} != {tuple(want.shape)}'
+    e = rel_err(got, want)
+    assert e == e and e < tol, f'{what}: relative error {e:.3e} is not below {tol:.1e}'
+    return e
+
+
+def assert_all_close(got, want, tol, what=''):
+    """`assert_close` over two equally long sequences of tensors; returns the list of errors."""
+    got, want = list(got), list(want)
+    assert len(got) == len(want), f'{what}: {len(got)} results, {len(want)} expected'
+    return [assert_close(a, b, tol, f'{what} #{i}') for i, (a, b) in enumerate(zip(got, want))]
+
+
 def loop_with_grads(step, inputs, states, douts, dstates, dtype=torch.float64):
     """Forward through `run_loop` and gradients of sum(<out,dout>) + sum(<stateT,dstate>)
     with respect to every input and initial state.  Returns (outs, final_states, dinputs, dstates0)."""
@@ -66,3 +91,45 @@ def loop_with_grads(step, inputs, states, douts, dstates, dtype=torch.float64):
     grads = torch.autograd.grad(ys, xs + ss, grad_outputs=gs, allow_unused=True)
     grads = [torch.zeros_like(p) if g is None else g for g, p in zip(grads, xs + ss)]
     return outs, fin, grads[:len(xs)], grads[len(xs):]
+
+
+def chunked_loop_with_grads(step, inputs, states, douts, dstates, chunk, dtype=torch.float64):
+    """Same results as `loop_with_grads`, holding the autograd graph of only `chunk` timesteps at
+    a time: a forward sweep without graph keeps the state at every chunk boundary; a reverse sweep
+    re-runs each chunk from its boundary state with a graph, differentiates
+    sum(<out_chunk, dout_chunk>) + <state at chunk end, its gradient> and hands the gradient of
+    the chunk's entry state to the chunk before.  Gradients of inputs without a time axis are
+    summed over the chunks.  Returns (outs, final_states, dinputs, dstates0)."""
+    T = max(x.shape[1] for x in inputs)
+    xs = [x.detach().to(dtype) for x in inputs]
+    timed = [x.shape[1] == T and T != 1 for x in xs]
+    bounds = list(range(0, T, chunk))
+    entry, outs_c = [], []
+    st = tuple(s.detach().to(dtype) for s in states)
+    with torch.no_grad():
+        for t0 in bounds:
+            entry.append(st)
+            sl = [x[:, t0:t0 + chunk] if td else x for x, td in zip(xs, timed)]
+            o, st = run_loop(step, sl, st, dtype)
+            outs_c.append(o)
+    outs = tuple(torch.cat([o[k] for o in outs_c], dim=1) for k in range(len(outs_c[0])))
+    fin = st
+    dins = [torch.zeros_like(x) for x in xs]
+    dst = [g.detach().to(dtype) for g in dstates]
+    gouts = [g.detach().to(dtype) for g in douts]
+    for ci in range(len(bounds) - 1, -1, -1):
+        t0 = bounds[ci]
+        sl = [(x[:, t0:t0 + chunk] if td else x).clone().requires_grad_() for x, td in zip(xs, timed)]
+        s_in = [s.clone().requires_grad_() for s in entry[ci]]
+        o, s_out = run_loop(step, sl, s_in, dtype)
+        ys = list(o) + list(s_out)
+        gs = [g[:, t0:t0 + chunk] for g in gouts] + list(dst)
+        grads = torch.autograd.grad(ys, sl + s_in, grad_outputs=gs, allow_unused=True)
+        grads = [torch.zeros_like(p) if g is None else g for g, p in zip(grads, sl + s_in)]
+        for i, td in enumerate(timed):
+            if td:
+                dins[i][:, t0:t0 + chunk] = grads[i]
+            else:
+                dins[i] += grads[i]
+        dst = [g.detach() for g in grads[len(sl):]]
+    return outs, fin, dins, dst

@@ -54,6 +54,19 @@ def _zoo2(x, g, c, S):
 
 CASES['zoo2'] = (_zoo2, [('row', 'BTH'), ('row', 'BT'), ('col', 'BTH')], 1)
 
+
+
+def _matgain(q, k, v, w, G, S):
+    """Gated linear attention with a per-element gain on the update: a matrix input whose gradient
+    does not read the state (it is formed by the per-chunk gradient kernel, not by the reverse scan)."""
+    S = S * th.sigmoid(w) + G * (v * k)
+    return (S * q).sum(-1, True), S
+
+
+CASES['matgain'] = (_matgain, [('row', 'BTH'), ('row', 'BTH'), ('col', 'BTH'), ('row', 'BTH'), ('mat', 'BH')], 1)
+# Mamba-1 with a decay matrix per (batch, head): a matrix input that is broadcast over nothing
+CASES['mamba_bh'] = (ops.mamba, [('col', 'BTH'), ('col', 'BTH'), ('mat', 'BH'), ('row', 'BT'), ('row', 'BT')], 1)
+
 # vector-state recurrences (N == 1)
 VECTOR_CASES = {
     'hgrn': (ops.hgrn, [('col', 'BT'), ('col', 'BT')], 1),
@@ -85,7 +98,7 @@ def make_inputs(name, B, T, H, M, N, dtype=th.float64, seed=0, table=None):
         xs[j] = th.sigmoid(xs[j].double()).to(dtype)
     if name == 'retention':
         xs[0] = th.sigmoid(xs[0].double() + 2).to(dtype)
-    if name in ('mamba', 'mamba2'):
+    if name in ('mamba', 'mamba2', 'mamba_bh'):
         xs[1] = F.softplus(xs[1].double() - 1).to(dtype)
         xs[2] = -th.sigmoid(xs[2].double()).to(dtype)
     if name == 's4d':

@@ -60,12 +60,9 @@ def main():
     want = recurrence.loop_with_grads(step, xs, ss, dyq, dSq)
     got = list(outs) + list(stT) + list(dins) + list(dst0)
     want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
-    worst = 0.0
-    for a, b in zip(got, want):
-        assert a.shape == b.shape, (a.shape, b.shape)
-        worst = max(worst, recurrence.rel_err(a, b))
+    print(f'{name} {dims} {dt} tile={plan.tile}', flush=True)
+    worst = max(recurrence.assert_all_close(got, want, tol, name))
     print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e}')
-    assert worst < tol, worst
 
 
 if __name__ == '__main__':

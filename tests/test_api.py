@@ -115,6 +115,30 @@ def test_dynamic_mode_plans_one_entry_per_signature():
     assert tuple(y.shape) == (2, 16, 2, 8)
 
 
+def test_dynamic_mode_backward_finds_the_plan_of_its_own_forward_call():
+    """Two signatures that differ only in the state's dtype (or only in its strides) have the same inputs
+    and checkpoint shapes.  The backward operator must still run the plan of the forward call it belongs to:
+    the hidden tag result carries the entry number in its shape."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    f = flex_rnn_amd.jit.dynamic(ops.delta_rule)
+    step, xs, ss = cases.make_inputs('delta_rule', 2, 16, 2, 8, 8, dtype=th.float32)
+    variants = [ss[0], ss[0].to(th.bfloat16), ss[0].transpose(-1, -2).contiguous().transpose(-1, -2)]
+    with FakeTensorMode() as mode:
+        fx = [mode.from_tensor(x) for x in xs]
+        outs = []
+        for s0 in variants:
+            fs = mode.from_tensor(s0).requires_grad_()
+            outs.append((fs, f(*fx, fs)))
+        assert len(f._entries) == 3 and sorted(f._by_id) == [1, 2, 3]
+        # backward of the calls in an order other than the forward calls'
+        for k in (0, 2, 1):
+            fs, (y, S) = outs[k]
+            (g,) = th.autograd.grad([y, S], [fs], [th.ones_like(y), th.ones_like(S)])
+            assert g.dtype == variants[k].dtype and g.stride() == variants[k].stride(), k
+    with pytest.raises(AssertionError, match='no forward call has produced'):
+        f._bw_entry(th.empty(0, 7, dtype=th.uint8))
+
+
 def test_infer_is_part_of_the_surface_and_has_no_cpu_fallback(runtime_lib):
     if th.cuda.is_available():
         pytest.skip('a GPU is present')

@@ -36,6 +36,13 @@ RUNS = [
     ('cfg:mamba2', '1,21,2,64,128', 'bf16', 0),
     ('rwkv4', '2,11,1,32,1', 'f32', 0),
     ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1),
+    # a single timestep with a matrix input that is broadcast over nothing: its gradient is still formed in
+    # fp32 (by the reverse scan for `mamba_bh`, by the gradient kernel for `matgain`) and cast afterwards
+    ('mamba_bh', '2,1,2,16,16', 'bf16', 1),
+    ('mamba_bh', '2,1,2,16,16', 'bf16', 0),
+    ('matgain', '2,1,2,16,16', 'bf16', 1),
+    ('matgain', '2,1,2,16,16', 'f16', 0),
+    ('matgain', '2,5,2,16,16', 'f64', 1),
     # the emitter's op table (sigmoid, tanh, softplus, where, relu, sqrt, rsqrt, log, min/max, ...)
     ('zoo', '2,8,2,16,16', 'f32', 1),
     ('zoo2', '2,8,2,16,16', 'f32', 0),

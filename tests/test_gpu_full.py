@@ -1,8 +1,8 @@
 """GPU tests at the benchmark sizes and of the calling conventions.
 
 The oracle (oracle/recurrence.py) is plain torch code, so for the full-size checks it runs on
-the GPU in fp64: forward over the whole sequence, and forward + gradients over a prefix of 128
-steps (autograd through the loop keeps every intermediate state alive).
+the GPU in fp64: forward over the whole sequence, and forward + gradients with its chunked
+backward (autograd through the whole loop would keep every intermediate state alive).
 """
 import pytest
 import torch as th
@@ -34,27 +34,32 @@ def test_full_size_forward_against_oracle(name):
     assert recurrence.rel_err(y, y_ref) < TOL[wl.dtype] and recurrence.rel_err(S, S_ref) < TOL[wl.dtype]
 
 
-@pytest.mark.parametrize('name', ['rwkv7', 'gated_delta_rule'])
-def test_full_width_gradients_against_oracle(name):
-    B, T, H, M, N = configs.DEFAULT_DIMS[name]
-    dims = (B, 128, H, M, N)
-    print(f'case full-width gradients {name} {dims}', flush=True)
-    wl = configs.make(name, dims=dims)
+@pytest.mark.parametrize('name,chunk', [('mamba1', 64), ('mamba2', 32), ('rwkv7', 32), ('gated_delta_rule', 64)])
+def test_full_size_outputs_states_and_gradients_against_oracle(name, chunk):
+    """The four GPU configurations at their full B, T, H, M, N: outputs, final state, the gradient of
+    every input (the atomically accumulated ones of inputs shared over batch, time or heads included)
+    and of the initial state against the oracle, which runs on the GPU in fp64 with its chunked
+    backward (autograd through `chunk` steps at a time; equal to the plain loop, tests/test_oracle.py)."""
+    dims = configs.DEFAULT_DIMS[name]
+    print(f'case full-size gradients {name} {dims}', flush=True)
+    wl = configs.make(name)
     dy, dS = configs.upstream_grads(wl)
     xs, ss = _gpu(wl.inputs), _gpu(wl.states)
     dyq = [g.cuda().to(wl.dtype) for g in dy]
     dSq = [g.cuda().to(wl.dtype) for g in dS]
-    want = recurrence.loop_with_grads(wl.step, xs, ss, dyq, dSq, dtype=th.float64)
-    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
     f = flex_rnn_amd.jit(wl.step)
-    xg = [x.requires_grad_() for x in xs]
-    sg = [s.requires_grad_() for s in ss]
+    xg = [x.clone().requires_grad_() for x in xs]
+    sg = [s.clone().requires_grad_() for s in ss]
     res = f(*xg, *sg)
     grads = th.autograd.grad(res, xg + sg, grad_outputs=dyq + dSq)
-    got = list(res) + list(grads)
-    errs = [recurrence.rel_err(a, b) for a, b in zip(got, want)]
+    got = [t.detach() for t in list(res) + list(grads)]
+    del res, grads, xg, sg
+    th.cuda.synchronize()
+    want = recurrence.chunked_loop_with_grads(wl.step, xs, ss, dyq, dSq, chunk, dtype=th.float64)
+    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    assert all(float(w.abs().max()) > 0 for w in want[2:])
+    errs = recurrence.assert_all_close(got, want, TOL[wl.dtype], name)
     print(['%.2e' % e for e in errs], flush=True)
-    assert max(errs) < TOL[wl.dtype]
 
 
 def test_chunked_call_equals_single_call_at_full_size():
@@ -162,6 +167,50 @@ def test_dynamic_mode_accepts_other_shapes():
         for a, b in zip(list(out) + list(grads), ref):
             assert recurrence.rel_err(a, b) < 1e-4, dims
     assert len(f._entries) == 3
+
+
+def test_dynamic_mode_signatures_that_differ_only_in_the_state():
+    """Same inputs and checkpoint shapes, the state once in fp32, once in bf16 and once transposed in
+    memory: three plans, and each backward call runs the plan of its own forward call (gradient of the
+    state in the state's dtype and layout), whatever the order of the backward calls."""
+    print('case dynamic state signatures', flush=True)
+    f = flex_rnn_amd.jit.dynamic(ops.gla)
+    step, xs, ss = cases.make_inputs('gla', 2, 16, 2, 16, 16, dtype=th.float32)
+    variants = [ss[0], ss[0].to(th.bfloat16), ss[0].transpose(-1, -2).contiguous().transpose(-1, -2)]
+    calls = []
+    for s0 in variants:
+        gx = [x.requires_grad_() for x in _gpu(xs)]
+        gs = s0.cuda().requires_grad_()
+        calls.append((gx, gs, f(*gx, gs)))
+    assert len(f._entries) == 3
+    g = th.Generator().manual_seed(5)
+    for k in (1, 2, 0):
+        gx, gs, out = calls[k]
+        dys = [th.randn(o.shape, generator=g).to(o.dtype) for o in out]
+        grads = th.autograd.grad(out, gx + [gs], [d.cuda() for d in dys])
+        assert grads[-1].dtype == variants[k].dtype and grads[-1].stride() == variants[k].stride()
+        want = recurrence.loop_with_grads(step, xs, [variants[k]], dys[:1], dys[1:], dtype=th.float64)
+        ref = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+        recurrence.assert_all_close(list(out) + list(grads), ref, 1e-2 if k == 1 else 1e-4, f'variant {k}')
+
+
+@pytest.mark.parametrize('name', ['mamba_bh', 'matgain'])
+def test_single_timestep_with_a_matrix_input_in_bf16(name):
+    """T = 1 and a matrix input that is broadcast over nothing: its gradient is accumulated in fp32 by the
+    kernels (reverse scan for `mamba_bh`, gradient kernel for `matgain`) and must come back in bf16."""
+    print(f'case T=1 matrix input {name}', flush=True)
+    step, xs, ss = cases.make_inputs(name, 2, 1, 2, 16, 16, dtype=th.bfloat16)
+    f = flex_rnn_amd.jit(step)
+    gx = [x.requires_grad_() for x in _gpu(xs)]
+    gs = [s_.requires_grad_() for s_ in _gpu(ss)]
+    out = f(*gx, *gs)
+    g = th.Generator().manual_seed(5)
+    dys = [th.randn(o.shape, generator=g).to(o.dtype) for o in out]
+    grads = th.autograd.grad(out, gx + gs, [d.cuda() for d in dys])
+    assert all(gr.dtype == th.bfloat16 and gr.shape == x.shape for gr, x in zip(grads, xs + ss))
+    want = recurrence.loop_with_grads(step, xs, ss, dys[:1], dys[1:], dtype=th.float64)
+    ref = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    recurrence.assert_all_close(list(out) + list(grads), ref, 1e-2, name)
 
 
 @pytest.mark.parametrize('name', ['rwkv7', 'mamba1', 'mamba2'])

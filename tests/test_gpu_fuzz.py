@@ -29,10 +29,7 @@ def test_random_recurrence(seed):
     want = recurrence.loop_with_grads(step, xs, ss, dout[:f.noutputs], dout[f.noutputs:])
     want = [*want[0], *want[1], *want[2], *want[3]]
     got = [o.detach().cpu() for o in out] + [th.zeros_like(x) if gr is None else gr.cpu() for gr, x in zip(grads, xs + ss)]
-    assert len(got) == len(want)
-    for i, (a, b) in enumerate(zip(got, want)):
-        assert a.shape == b.shape
-        assert recurrence.rel_err(a, b) < TOL[dtype], (i, recurrence.rel_err(a, b))
+    recurrence.assert_all_close(got, want, TOL[dtype], f'seed {seed}')
     # the inference kernel agrees with the training forward
     lean = f.infer(*[x.cuda() for x in xs], *[s.cuda() for s in ss])
     for a, b in zip(lean, out):

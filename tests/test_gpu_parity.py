@@ -29,9 +29,7 @@ def run_case(name, dims, dtype, seed=0):
     grads = th.autograd.grad(res, xs + ss, grad_outputs=[g.cuda().to(r.dtype) for g, r in zip(dy + dS, res)])
     th.cuda.synchronize()
     got = list(res) + list(grads)
-    errs = [recurrence.rel_err(a, b) for a, b in zip(got, want)]
-    for a, b in zip(got, want):
-        assert a.shape == b.shape
+    errs = recurrence.assert_all_close(got, want, TOL[wl.dtype], f'{name} {dims}')
     return errs, got, wl
 
 
@@ -65,5 +63,4 @@ def test_committed_vectors(name):
     res = flex_rnn_amd.jit(step)(*xs, *ss)
     grads = th.autograd.grad(res, xs + ss, [g.float().cuda() for g in arrs('dy') + arrs('dS')])
     want = arrs('out') + arrs('stT') + arrs('din') + arrs('dst')
-    errs = [recurrence.rel_err(a, b) for a, b in zip(list(res) + list(grads), want)]
-    assert max(errs) < 1e-4, errs
+    recurrence.assert_all_close(list(res) + list(grads), want, 1e-4, f'golden {name}')

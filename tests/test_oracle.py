@@ -185,3 +185,88 @@ def test_committed_vectors(name):
     naive = flex_rnn_amd.jit(step).naive(*xs, *ss, dtype=th.float64)
     for a, b in zip(naive, arrs('out') + arrs('stT')):
         assert recurrence.rel_err(a, b) < 1e-12
+
+
+# ------------------------------------------------------------------ the metric and the assertion
+def test_rel_err_known_values():
+    """||a - b|| / max(||b||, 1e-30) with b the trusted value (check_grad.py:20)."""
+    import math
+    a, b = th.tensor([3.0, 4.0]), th.tensor([0.0, 5.0])
+    # a - b = (3, -1): sqrt(10) / 5.  (Squared norms would give 0.4, dividing by ||a|| the same 0.632 only
+    # by accident of |a| = |b| = 5, which the next pair tells apart.)
+    assert recurrence.rel_err(a, b) == pytest.approx(math.sqrt(10) / 5, rel=1e-15)
+    a2, b2 = th.tensor([6.0, 8.0]), th.tensor([0.0, 5.0])
+    assert recurrence.rel_err(a2, b2) == pytest.approx(math.sqrt(45) / 5, rel=1e-15)       # divided by ||b|| = 5 ...
+    assert recurrence.rel_err(b2, a2) == pytest.approx(math.sqrt(45) / 10, rel=1e-15)      # ... not by ||a|| = 10
+    # a zero reference: the 1e-30 floor, no division by zero
+    assert recurrence.rel_err(th.zeros(4), th.zeros(4)) == 0.0
+    assert recurrence.rel_err(th.tensor([2e-30, 0.0]), th.zeros(2)) == pytest.approx(2.0, rel=1e-6)
+    # identical tensors of any dtype and shape
+    x = th.randn(3, 5, dtype=th.bfloat16)
+    assert recurrence.rel_err(x, x) == 0.0
+    # operands are promoted to double before subtracting: 1 + 2^-10 is not a bf16 number (nearest: 1), so
+    # a bf16 subtraction of the promoted-late kind would see no difference at all
+    one = th.ones(1, dtype=th.bfloat16)
+    assert recurrence.rel_err(one, th.tensor([1.0 + 2.0 ** -10], dtype=D)) == pytest.approx(2.0 ** -10 / (1 + 2.0 ** -10), rel=1e-12)
+    # and a difference far below float32 resolution survives (no .float() on the way)
+    assert recurrence.rel_err(th.tensor([1.0 + 1e-13], dtype=D), th.tensor([1.0], dtype=D)) == pytest.approx(1e-13, rel=1e-2)
+    # the whole tensor enters, not the worst element and not the mean
+    assert recurrence.rel_err(th.tensor([1.0, 1.0, 1.0, 2.0]), th.ones(4)) == pytest.approx(0.5, rel=1e-15)
+
+
+@pytest.mark.parametrize('tol', [1e-4, 1e-2])
+def test_assert_close_rejects_twice_the_tolerance(tol):
+    """Negative test of the assertion the GPU parity tests use: a result whose error is 2 x tol fails, one
+    at tol / 2 passes; wrong shapes, NaNs and a wrong count fail."""
+    want = rnd(4, 7, 3, seed=1)
+    noise = rnd(4, 7, 3, seed=2)
+    noise = noise / noise.norm() * want.norm()          # relative size exactly 1
+    ok = want + 0.5 * tol * noise
+    bad = want + 2.0 * tol * noise
+    assert recurrence.assert_close(ok, want, tol) == pytest.approx(0.5 * tol, rel=1e-6)
+    with pytest.raises(AssertionError, match='relative error'):
+        recurrence.assert_close(bad, want, tol)
+    with pytest.raises(AssertionError, match='relative error'):
+        recurrence.assert_all_close([ok, bad], [want, want], tol)
+    assert recurrence.assert_all_close([ok, want], [want, want], tol)[1] == 0.0
+    with pytest.raises(AssertionError, match='shape'):
+        recurrence.assert_close(want[:, :, :2], want, tol)
+    with pytest.raises(AssertionError, match='shape'):
+        recurrence.assert_close(want.reshape(7, 4, 3), want, tol)
+    nan = want.clone()
+    nan[0, 0, 0] = float('nan')
+    with pytest.raises(AssertionError):
+        recurrence.assert_close(nan, want, tol)
+    with pytest.raises(AssertionError, match='expected'):
+        recurrence.assert_all_close([want], [want, want], tol)
+    # a dropped contribution (one timestep's share of a sum) and a doubled one are both far outside
+    parts = [rnd(5, 6, seed=10 + i) for i in range(16)]
+    total = sum(parts)
+    with pytest.raises(AssertionError):
+        recurrence.assert_close(total - parts[3], total, tol)
+    with pytest.raises(AssertionError):
+        recurrence.assert_close(total + parts[3], total, tol)
+
+
+# ------------------------------------------------------------------ chunked backward
+@pytest.mark.parametrize('name,dims,chunk', [
+    ('rwkv7', (2, 12, 2, 4, 4), 4), ('rwkv7', (1, 13, 2, 4, 8), 5), ('gated_delta_rule', (2, 9, 1, 4, 4), 2),
+    ('mamba', (2, 10, 2, 4, 4), 3), ('mamba2', (2, 8, 3, 4, 4), 8), ('s4d', (2, 7, 1, 4, 4), 3),
+    ('rwkv6', (2, 6, 2, 4, 4), 1), ('rwkv4', (2, 11, 1, 8, 1), 4), ('mlstm_gates', (2, 5, 2, 4, 1), 16)])
+def test_chunked_backward_equals_unchunked(name, dims, chunk):
+    """`chunked_loop_with_grads` == `loop_with_grads` in fp64 (1e-12): outputs, final states, every input
+    gradient (time-broadcast and matrix inputs, summed over chunks, included) and the initial-state
+    gradients; chunk lengths that divide T, that do not, of one step, and longer than T."""
+    import cases
+    step, xs, ss = cases.make_inputs(name, *dims, dtype=D)
+    g = th.Generator().manual_seed(7)
+    outs, fin = recurrence.run_loop(step, xs, ss)
+    dy = [th.randn(o.shape, generator=g, dtype=D) for o in outs]
+    dS = [th.randn(s.shape, generator=g, dtype=D) for s in fin]
+    a = recurrence.loop_with_grads(step, xs, ss, dy, dS)
+    b = recurrence.chunked_loop_with_grads(step, xs, ss, dy, dS, chunk)
+    for part_a, part_b in zip(a, b):
+        errs = recurrence.assert_all_close(part_b, part_a, 1e-12, name)
+        assert len(errs) == len(part_a)
+    # the gradients are not trivially zero (a chunked sweep that dropped the state hand-off would still pass then)
+    assert all(float(g_.abs().max()) > 0 for g_ in b[3])

@@ -64,15 +64,18 @@ def warm(force=False, seen=None):
         step, xs, ss = cases.make_inputs('gla', 2, 32, 2, 32, 32, dtype=dtype)
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
         plans.append(plan)
+    for name in ('mamba_bh', 'matgain'):                # a single timestep with a full matrix input, bf16
+        step, xs, ss = cases.make_inputs(name, 2, 1, 2, 16, 16, dtype=th.bfloat16)
+        plans.append(planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0])
+    step, xs, ss = cases.make_inputs('gla', 2, 16, 2, 16, 16, dtype=th.float32)      # state dtype / layout variants
+    for s0 in (ss[0], ss[0].to(th.bfloat16), ss[0].transpose(-1, -2).contiguous().transpose(-1, -2)):
+        plans.append(planner.make_plan(step, [x.to('meta') for x in xs], [s0.to('meta')])[0])
     for seed in cases.FUZZ_SEEDS:                       # tests/test_gpu_fuzz.py
         step, xs, ss = cases.fuzz_case(seed, (th.float32, th.bfloat16)[(seed // 6) % 2])
         plan = planner.make_plan(step, [x.to('meta') for x in xs], [s.to('meta') for s in ss])[0]
         plans.append(plan)
     for name, dims in GOLDEN.items():
         plans.append(prebuild.plan_for(name, dims, th.float32))
-    for name in ('rwkv7', 'gated_delta_rule'):
-        B, T, H, M, N = configs.DEFAULT_DIMS[name]
-        plans.append(prebuild.plan_for(name, (B, 128, H, M, N)))
     plans.append(prebuild.plan_for('rwkv7', (8, 512, 32, 128, 128)))
     plans.append(prebuild.plan_for('mamba2', (2, 64, 4, 64, 128)))
     for name in ('rwkv7', 'mamba1', 'mamba2'):
