@@ -36,28 +36,14 @@ PUBLISHED_TOKENS_PER_S = {'rwkv7': 8192 / 55e-3}
 PUBLISHED_NOTE = 'reference README: 55 ms per fwd+bwd step on an RTX 4070 mobile (other hardware)'
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
-    ap.add_argument('--warmup', type=int, default=5)
-    ap.add_argument('--workload', default='rwkv7', choices=sorted(WORK))
-    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
-    ap.add_argument('--calibrate-copy', action='store_true',
-                    help='also run one plain 1 GiB device copy (reference dispatch for HBM byte counters)')
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f'bench.py: this build measures one GPU; --gpus {args.gpus} is not supported '
-              '(the recurrence shards over batch x head with no exchange between GPUs; each GPU would run this same path).', file=sys.stderr)
-        sys.exit(2)
-
+def measure(name, steps, warmup, traffic_records):
+    """`steps` timed forward + backward passes of workload `name` at its full size (inputs resident in HBM).
+    Returns (result fields, the compiled plan)."""
     import torch as th
     import flex_rnn_amd
-    from flex_rnn_amd import configs, launch
+    from flex_rnn_amd import configs, runtime
 
-    assert th.cuda.is_available(), 'bench.py needs a GPU'
     dev = th.device('cuda:0')
-    name = args.workload
     wl = configs.make(name, device='cpu')
     B, T, H, M, N = wl.dims
     dy, dS = configs.upstream_grads(wl)
@@ -73,14 +59,14 @@ def main():
             gy = [g.to(dev).to(r.dtype) for g, r in zip(dy + dS, res)]
         return th.autograd.grad(res, xs + ss, grad_outputs=gy)
 
-    for _ in range(max(args.warmup, 1)):
+    for _ in range(max(warmup, 1)):
         step()
     th.cuda.synchronize()
     compiled = f.forward_func.compiled
     compiled.profile_events = []
     th.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step()
     th.cuda.synchronize()
     wall = time.perf_counter() - t0
@@ -92,22 +78,22 @@ def main():
             f(*xs, *ss)
         th.cuda.synchronize()
         t1 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             f(*xs, *ss)
         th.cuda.synchronize()
-        fwd_ms = (time.perf_counter() - t1) * 1e3 / args.steps
+        fwd_ms = (time.perf_counter() - t1) * 1e3 / steps
         # inference: the forward kernel that saves nothing for a backward pass
         for _ in range(2):
             f.infer(*xs, *ss)
         th.cuda.synchronize()
         t1 = time.perf_counter()
-        for _ in range(args.steps):
+        for _ in range(steps):
             f.infer(*xs, *ss)
         th.cuda.synchronize()
-        inf_ms = (time.perf_counter() - t1) * 1e3 / args.steps
-    ms_per_step = wall * 1e3 / args.steps
+        inf_ms = (time.perf_counter() - t1) * 1e3 / steps
+    ms_per_step = wall * 1e3 / steps
     tokens = B * T
-    value = tokens / (wall / args.steps)
+    value = tokens / (wall / steps)
 
     per = {}
     for kname, e0, e1 in ev:
@@ -124,16 +110,23 @@ def main():
     achieved = kflop[dominant] * elems / (kavg[dominant] * 1e-3) / 1e12
     gpu_ms = sum(kavg.values())
     step_tflops = (w['flop_fwd'] + w['flop_bwd']) * elems / (gpu_ms * 1e-3) / 1e12
-    traffic = None        # HBM bytes per launch of the dominant kernel, from the committed rocprofv3 --pmc runs
-    tpath = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
-    if os.path.isfile(tpath):
-        rec = json.load(open(tpath)).get(name, {}).get(dominant)
-        if rec:
-            traffic = round(rec['read_bytes'] + rec['write_bytes'])
+    # HBM bytes per launch come from committed rocprofv3 --pmc runs (profiles/hbm_traffic.json), each recorded with
+    # the cache key of the kernel source it was taken on: a figure for another build of the kernel is not reported
+    keys = {k: runtime.source_key(spec.name, spec.source) for k, (spec, _) in compiled.kernels.items()}
+
+    def traffic_of(kernels):
+        recs = traffic_records.get(name, {})
+        if all(k in recs and recs[k].get('kernel_key') == keys[k] for k in kernels):
+            return round(sum(recs[k]['read_bytes'] + recs[k]['write_bytes'] for k in kernels))
+        return None
+
+    traffic = traffic_of([dominant])
     hbm_gbps = w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9
     roofline = {
         'bound': 'valu', 'kernel': dominant, 'achieved': round(achieved, 3), 'peak': PEAK_FP32_TFLOPS,
         'unit': 'TFLOP/s', 'frac': round(achieved / PEAK_FP32_TFLOPS, 4), 'traffic': traffic,
+        'traffic_source': ('profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this kernel build)'
+                           if traffic is not None else 'none: no committed counter run for the kernel build that ran'),
         'kernel_ms': {k: round(v, 4) for k, v in kavg.items()},
         'step_achieved': round(step_tflops, 3), 'step_frac': round(step_tflops / PEAK_FP32_TFLOPS, 4),
         'hbm_GBps_algorithmic': round(hbm_gbps, 1), 'hbm_frac': round(hbm_gbps / PEAK_HBM_GBS, 4),
@@ -142,15 +135,72 @@ def main():
     # small state rows, so the per-token vectors outweigh the arithmetic), the algorithmic bytes of a pass do not
     # split between the two backward kernels, so the figure is quoted for the three kernels of the step together.
     if w['bytes_all'] * tokens / (PEAK_HBM_GBS * 1e9) > (w['flop_fwd'] + w['flop_bwd']) * elems / (PEAK_FP32_TFLOPS * 1e12):
-        if traffic is not None:
-            recs = json.load(open(tpath))[name]
-            traffic = round(sum(r['read_bytes'] + r['write_bytes'] for k, r in recs.items() if k in kavg))
+        traffic = traffic_of(sorted(kavg))
         roofline.update({'bound': 'hbm', 'kernel': '+'.join(sorted(kavg)), 'achieved': round(hbm_gbps, 1),
                          'peak': PEAK_HBM_GBS, 'unit': 'GB/s', 'frac': round(hbm_gbps / PEAK_HBM_GBS, 4),
                          'traffic': traffic, 'valu_TFLOPs_algorithmic': round(step_tflops, 3),
                          'valu_frac': round(step_tflops / PEAK_FP32_TFLOPS, 4)})
+        if traffic is None:
+            roofline['traffic_source'] = 'none: no committed counter run for the kernel builds that ran'
         for k in ('step_achieved', 'step_frac', 'hbm_GBps_algorithmic', 'hbm_frac'):
             del roofline[k]
+
+    def finite(v):
+        return None if v is None or v != v or v in (float('inf'), float('-inf')) else round(v, 4)
+
+    res = {
+        'value': round(value, 1), 'ms_per_step': round(ms_per_step, 4),
+        'io_dtype': str(wl.dtype).replace('torch.', ''),
+        'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
+        'roofline': roofline,
+        'gpu_kernel_ms_per_step': round(gpu_ms, 4),
+        'gpu_kernel_ms_per_step_quantiles': quantiles,
+        'kernel_keys': keys,
+        'forward_only': {'ms_per_step': round(fwd_ms, 4), 'tokens_per_s': round(tokens / (fwd_ms * 1e-3), 1),
+                         'achieved_TFLOPs': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12, 3),
+                         'frac': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4)},
+        'inference': {'ms_per_step': round(inf_ms, 4), 'tokens_per_s': round(tokens / (inf_ms * 1e-3), 1)},
+    }
+    from flex_rnn_amd import launch
+    # candidate builds of each kernel as timed on the first call of this device (the fastest runs; the choice is kept
+    # beside the kernel cache, so a later process reports the stored timings)
+    res['row_kernel_builds'] = {k: {'tiles (L, C, R, W)': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
+                                    'ms': compiled.build_times.get(k) and [finite(v) for v in compiled.build_times[k]]}
+                                for k in ('frnn_fw', 'frnn_bw1')}
+    bt = compiled.bw2_times
+    res['gradient_kernel_builds'] = [
+        {'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
+         'ms': finite(bt[i]) if bt and i < len(bt) else None}
+        for i, (_, _, r) in enumerate(compiled.bw2_builds)]
+    del xs, ss, gy, f
+    th.cuda.empty_cache()
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--workload', default='rwkv7', choices=sorted(WORK))
+    ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
+    ap.add_argument('--no-others', action='store_true', help='skip the short runs of the other three GPU workloads')
+    ap.add_argument('--calibrate-copy', action='store_true',
+                    help='also run one plain 1 GiB device copy (reference dispatch for HBM byte counters)')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f'bench.py: this build measures one GPU; --gpus {args.gpus} is not supported '
+              '(the recurrence shards over batch x head with no exchange between GPUs; each GPU would run this same path).', file=sys.stderr)
+        sys.exit(2)
+
+    import torch as th
+
+    assert th.cuda.is_available(), 'bench.py needs a GPU'
+    dev = th.device('cuda:0')
+    name = args.workload
+    tpath = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+    traffic_records = json.load(open(tpath)) if os.path.isfile(tpath) else {}
+    head = measure(name, args.steps, args.warmup, traffic_records)
 
     if args.calibrate_copy:
         src = th.empty(1 << 28, dtype=th.float32, device=dev).normal_()
@@ -158,35 +208,37 @@ def main():
         dst.copy_(src)                      # reads 1 GiB, writes 1 GiB
         th.cuda.synchronize()
         del src, dst
+    # the other GPU workloads, a few steps each: ms per step, tokens/s, binding roofline and fraction, per-kernel ms
+    others = None
+    if name == 'rwkv7' and not args.no_others:
+        others = {}
+        for other in ('mamba1', 'mamba2', 'gated_delta_rule'):
+            r = measure(other, 5, 2, traffic_records)
+            rf = r['roofline']
+            others[other] = {'workload': r['config']['workload'], 'ms_per_step': r['ms_per_step'], 'tokens_per_s': r['value'],
+                             'steps': 5, 'warmup': 2, 'bound': rf['bound'], 'frac': rf['frac'] if rf['bound'] == 'hbm' else rf['step_frac'],
+                             'frac_of': 'algorithmic HBM bytes of the step / 8 TB/s' if rf['bound'] == 'hbm'
+                             else 'algorithmic flops of the step / 157.3 TFLOP/s',
+                             'dominant_kernel': rf['kernel'], 'dominant_kernel_frac': rf['frac'],
+                             'kernel_ms': rf['kernel_ms'], 'gpu_kernel_ms_per_step': r['gpu_kernel_ms_per_step']}
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(name)
 
     out = {
-        'metric': 'fwd+bwd tokens/sec', 'value': round(value, 1), 'unit': 'tokens/s', 'n_gpus': 1,
-        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'metric': 'fwd+bwd tokens/sec', 'value': head['value'], 'unit': 'tokens/s', 'n_gpus': 1,
+        'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': head['ms_per_step'],
         'higher_is_better': True, 'scaling': 'weak',
-        'vs_baseline': round(value / PUBLISHED_TOKENS_PER_S[name], 2) if name in PUBLISHED_TOKENS_PER_S else None,
+        'vs_baseline': round(head['value'] / PUBLISHED_TOKENS_PER_S[name], 2) if name in PUBLISHED_TOKENS_PER_S else None,
         'baseline_note': PUBLISHED_NOTE if name in PUBLISHED_TOKENS_PER_S else None,
-        'dtype': 'f32',
-        'io_dtype': str(wl.dtype).replace('torch.', ''), 'data': 'synthetic',
-        'config': {'workload': f'{name} B{B} T{T} H{H} M{M} N{N} {str(wl.dtype).replace("torch.", "")} I/O, fwd+bwd'},
-        'roofline': roofline, 'cpu_baseline': cpu,
-        'gpu_kernel_ms_per_step': round(gpu_ms, 4),
-        'gpu_kernel_ms_per_step_quantiles': quantiles,
-        # candidate builds of the gradient kernel as timed on the first backward call (the fastest runs)
-        'row_kernel_builds': {k: {'tiles (L, C, R, W)': launch.row_kernel_tiles(compiled.plan, k == 'frnn_bw1'),
-                                  'ms': compiled.build_times.get(k) and [round(v, 4) for v in compiled.build_times[k]]}
-                              for k in ('frnn_fw', 'frnn_bw1')},
-        'gradient_kernel_builds': [
-            {'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
-             'ms': compiled.bw2_times and round(compiled.bw2_times[i], 4)}
-            for i, (_, _, r) in enumerate(compiled.bw2_builds)],
-        'forward_only': {'ms_per_step': round(fwd_ms, 4), 'tokens_per_s': round(tokens / (fwd_ms * 1e-3), 1),
-                         'achieved_TFLOPs': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12, 3),
-                         'frac': round(w['flop_fwd'] * elems / (fwd_ms * 1e-3) / 1e12 / PEAK_FP32_TFLOPS, 4)},
-        'inference': {'ms_per_step': round(inf_ms, 4), 'tokens_per_s': round(tokens / (inf_ms * 1e-3), 1)},
+        'dtype': 'f32', 'io_dtype': head['io_dtype'], 'data': 'synthetic',
+        'config': head['config'], 'roofline': head['roofline'], 'cpu_baseline': cpu,
     }
+    for k in ('gpu_kernel_ms_per_step', 'gpu_kernel_ms_per_step_quantiles', 'kernel_keys', 'row_kernel_builds',
+              'gradient_kernel_builds', 'forward_only', 'inference'):
+        out[k] = head[k]
+    if others is not None:
+        out['other_workloads'] = others
     print(json.dumps(out))
 
 

@@ -4,6 +4,7 @@
 // (dlsym(RTLD_DEFAULT)) so that the copy PyTorch already loaded is the one used, and is
 // dlopen'ed by soname only when the process has none.
 #include "frnn_rt.h"
+#include "frnn_internal.h"
 
 #include <dlfcn.h>
 #include <errno.h>
@@ -37,6 +38,8 @@ int fail(int code, const char* fmt, ...) {
   g_err = buf;
   return code;
 }
+
+void set_error(const char* msg) { g_err = msg; }
 
 // ---------------------------------------------------------------- HIP entry points
 typedef int hipError_t;
@@ -157,10 +160,181 @@ std::vector<std::string> split_ws(const char* s) {
 
 }  // namespace
 
+int frnn_detail_fail(int code, const char* fmt, ...) {
+  char buf[4096];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  set_error(buf);
+  return code;
+}
+
 struct frnn_module_s {
   void* mod;
   std::vector<char> image;   // the code object bytes; kept for the lifetime of the module
+  std::vector<frnn_kernel_s*> kernels;   // handles given out by frnn_get_kernel; freed with the module
 };
+
+namespace {
+
+// ---------------------------------------------------------------- code object metadata
+// The AMDGPU metadata note of a code object is a MessagePack map
+//   { "amdhsa.kernels": [ { ".name": <str>, ".kernarg_segment_size": <uint>, ... }, ... ], ... }.
+// Only what is needed to read that one number is implemented.
+struct MsgPack {
+  const uint8_t* p;
+  const uint8_t* e;
+  bool ok = true;
+
+  uint64_t be(int n) {
+    if (e - p < n) { ok = false; return 0; }
+    uint64_t v = 0;
+    for (int i = 0; i < n; i++) v = (v << 8) | *p++;
+    return v;
+  }
+  bool str(const char** s, size_t* n) {         // consumes a string; false (nothing consumed) for another type
+    if (p >= e) return ok = false;
+    const uint8_t t = *p;
+    const uint8_t* save = p;
+    size_t len;
+    if (t >= 0xa0 && t <= 0xbf) { len = t & 0x1f; p++; }
+    else if (t == 0xd9 || t == 0xda || t == 0xdb) { p++; len = (size_t)be(t == 0xd9 ? 1 : t == 0xda ? 2 : 4); }
+    else return false;
+    if (!ok || (size_t)(e - p) < len) { p = save; return ok = false; }
+    *s = (const char*)p; *n = len; p += len;
+    return true;
+  }
+  bool uint_(uint64_t* v) {
+    if (p >= e) return ok = false;
+    uint8_t t = *p;
+    if (t <= 0x7f) { *v = t; p++; return true; }
+    if (t >= 0xcc && t <= 0xcf) { p++; *v = be(1 << (t - 0xcc)); return ok; }
+    if (t >= 0xd0 && t <= 0xd3) { p++; *v = be(1 << (t - 0xd0)); return ok; }
+    return false;
+  }
+  bool container(uint8_t fix_lo, uint8_t t16, size_t* n) {     // map or array header
+    if (p >= e) return ok = false;
+    uint8_t t = *p;
+    if (t >= fix_lo && t <= fix_lo + 0x0f) { *n = t & 0x0f; p++; return true; }
+    if (t == t16) { p++; *n = (size_t)be(2); return ok; }
+    if (t == t16 + 1) { p++; *n = (size_t)be(4); return ok; }
+    return false;
+  }
+  bool map(size_t* n) { return container(0x80, 0xde, n); }
+  bool array(size_t* n) { return container(0x90, 0xdc, n); }
+  void skip(int depth = 0) {
+    if (!ok || p >= e || depth > 64) { ok = false; return; }
+    size_t n;
+    const char* s;
+    uint64_t v;
+    uint8_t t = *p;
+    if (map(&n)) { for (size_t i = 0; i < 2 * n && ok; i++) skip(depth + 1); return; }
+    if (array(&n)) { for (size_t i = 0; i < n && ok; i++) skip(depth + 1); return; }
+    if (str(&s, &n) || uint_(&v)) return;
+    if (!ok) return;
+    p++;
+    if (t == 0xc0 || t == 0xc2 || t == 0xc3 || t >= 0xe0) return;                 // nil, bool, negative fixint
+    if (t == 0xca) { be(4); return; }
+    if (t == 0xcb) { be(8); return; }
+    if (t >= 0xc4 && t <= 0xc6) { size_t len = (size_t)be(1 << (t - 0xc4)); if ((size_t)(e - p) < len) ok = false; else p += len; return; }
+    if (t >= 0xd4 && t <= 0xd8) { be(1 + (1 << (t - 0xd4))); return; }           // fixext
+    if (t >= 0xc7 && t <= 0xc9) { size_t len = (size_t)be(1 << (t - 0xc7)); be(1); if ((size_t)(e - p) < len) ok = false; else p += len; return; }
+    ok = false;
+  }
+};
+
+bool key_is(const char* s, size_t n, const char* lit) { return n == strlen(lit) && memcmp(s, lit, n) == 0; }
+
+// kernarg segment size of `kernel` from an AMDGPU metadata blob; 0 when not found
+size_t kernarg_from_metadata(const uint8_t* d, size_t len, const char* kernel) {
+  MsgPack m{d, d + len};
+  size_t n;
+  if (!m.map(&n)) return 0;
+  for (size_t i = 0; i < n && m.ok; i++) {
+    const char* k; size_t kn;
+    if (!m.str(&k, &kn)) return 0;
+    if (!key_is(k, kn, "amdhsa.kernels")) { m.skip(); continue; }
+    size_t nk;
+    if (!m.array(&nk)) return 0;
+    for (size_t j = 0; j < nk && m.ok; j++) {
+      size_t nf;
+      if (!m.map(&nf)) return 0;
+      bool mine = false;
+      uint64_t size = 0;
+      for (size_t f = 0; f < nf && m.ok; f++) {
+        const char* fk; size_t fkn;
+        if (!m.str(&fk, &fkn)) return 0;
+        if (key_is(fk, fkn, ".name")) {
+          const char* v; size_t vn;
+          if (!m.str(&v, &vn)) return 0;
+          mine = key_is(v, vn, kernel);
+        } else if (key_is(fk, fkn, ".kernarg_segment_size")) {
+          if (!m.uint_(&size)) return 0;
+        } else {
+          m.skip();
+        }
+      }
+      if (mine && m.ok) return (size_t)size;
+    }
+    return 0;
+  }
+  return 0;
+}
+
+// The gfx ELF inside `image` (an ELF itself, or an uncompressed clang offload bundle holding one).
+bool find_device_elf(const std::vector<char>& image, const uint8_t** elf, size_t* len) {
+  const uint8_t* b = (const uint8_t*)image.data();
+  size_t n = image.size();
+  static const char kBundle[] = "__CLANG_OFFLOAD_BUNDLE__";
+  if (n > 64 && memcmp(b, "\177ELF", 4) == 0) { *elf = b; *len = n; return true; }
+  if (n < 32 || memcmp(b, kBundle, sizeof kBundle - 1) != 0) return false;
+  uint64_t count;
+  memcpy(&count, b + 24, 8);
+  size_t off = 32;
+  for (uint64_t i = 0; i < count && i < 64; i++) {
+    if (off + 24 > n) return false;
+    uint64_t eo, es, tl;
+    memcpy(&eo, b + off, 8); memcpy(&es, b + off + 8, 8); memcpy(&tl, b + off + 16, 8);
+    off += 24;
+    if (tl > n || off + tl > n) return false;
+    bool device = tl >= 3 && memcmp(b + off, "hip", 3) == 0;
+    off += tl;
+    if (device && es > 64 && eo <= n && es <= n - eo && memcmp(b + eo, "\177ELF", 4) == 0) { *elf = b + eo; *len = (size_t)es; return true; }
+  }
+  return false;
+}
+
+// 0 when the image has no readable metadata for `kernel` (the launch check is then skipped)
+size_t kernarg_segment_size(const std::vector<char>& image, const char* kernel) {
+  const uint8_t* e; size_t n;
+  if (!find_device_elf(image, &e, &n) || n < 64 || e[4] != 2 /*ELFCLASS64*/ || e[5] != 1 /*little endian*/) return 0;
+  uint64_t shoff; uint16_t shentsize, shnum;
+  memcpy(&shoff, e + 0x28, 8); memcpy(&shentsize, e + 0x3a, 2); memcpy(&shnum, e + 0x3c, 2);
+  if (shentsize < 64 || shoff > n || (uint64_t)shnum * shentsize > n - shoff) return 0;
+  for (unsigned i = 0; i < shnum; i++) {
+    const uint8_t* sh = e + shoff + (uint64_t)i * shentsize;
+    uint32_t type; uint64_t off, size;
+    memcpy(&type, sh + 4, 4); memcpy(&off, sh + 0x18, 8); memcpy(&size, sh + 0x20, 8);
+    if (type != 7 /*SHT_NOTE*/ || off > n || size > n - off) continue;
+    const uint8_t* p = e + off; const uint8_t* end = p + size;
+    while ((size_t)(end - p) >= 12) {
+      uint32_t namesz, descsz, ntype;
+      memcpy(&namesz, p, 4); memcpy(&descsz, p + 4, 4); memcpy(&ntype, p + 8, 4);
+      p += 12;
+      size_t na = ((size_t)namesz + 3) & ~(size_t)3, da = ((size_t)descsz + 3) & ~(size_t)3;
+      if (na > (size_t)(end - p) || da > (size_t)(end - p) - na) break;
+      if (ntype == 32 /*NT_AMDGPU_METADATA*/ && namesz == 7 && memcmp(p, "AMDGPU", 6) == 0) {
+        size_t r = kernarg_from_metadata(p + na, descsz, kernel);
+        if (r) return r;
+      }
+      p += na + da;
+    }
+  }
+  return 0;
+}
+
+}  // namespace
 
 extern "C" {
 
@@ -250,7 +424,7 @@ int frnn_module_load(const char* path, frnn_module_t* out) {
   fseek(f, 0, SEEK_END);
   long n = ftell(f);
   fseek(f, 0, SEEK_SET);
-  frnn_module_s* m = new frnn_module_s{nullptr, std::vector<char>((size_t)(n > 0 ? n : 0))};
+  frnn_module_s* m = new frnn_module_s{nullptr, std::vector<char>((size_t)(n > 0 ? n : 0)), {}};
   size_t got = n > 0 ? fread(m->image.data(), 1, (size_t)n, f) : 0;
   fclose(f);
   if (n <= 0 || got != (size_t)n) {
@@ -281,7 +455,15 @@ int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out) {
   void* fn = nullptr;
   hipError_t e = h.ModuleGetFunction(&fn, m->mod, name);
   if (e != 0) return hip_fail("hipModuleGetFunction", e);
-  *out = fn;
+  frnn_kernel_s* k = new frnn_kernel_s{fn, kernarg_segment_size(m->image, name)};
+  m->kernels.push_back(k);
+  *out = k;
+  return FRNN_OK;
+}
+
+int frnn_kernel_arg_bytes(frnn_kernel_t k, size_t* out) {
+  if (!k || !out) return fail(FRNN_ERR_ARG, "frnn_kernel_arg_bytes: null argument");
+  *out = k->kernarg;
   return FRNN_OK;
 }
 
@@ -298,10 +480,12 @@ int frnn_launch(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3]
   // this project take 8-byte fields only, so anything else is a packing mistake (a short block
   // leaves the kernel reading arguments that were never set).
   if (arg_bytes % 8 != 0) return fail(FRNN_ERR_ARG, "frnn_launch: argument block must be a whole number of 8-byte words");
+  if (k->kernarg && arg_bytes != k->kernarg)
+    return fail(FRNN_ERR_ARG, "frnn_launch: argument block of %zu bytes, the kernel's code object declares %zu", arg_bytes, k->kernarg);
   size_t sz = arg_bytes;
   void* extra[] = {(void*)0x01 /*BUFFER_POINTER*/, const_cast<void*>(args), (void*)0x02 /*BUFFER_SIZE*/, &sz,
                    (void*)0x03 /*END*/};
-  hipError_t e = h.ModuleLaunchKernel(k, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, stream,
+  hipError_t e = h.ModuleLaunchKernel(k->fn, grid[0], grid[1], grid[2], block[0], block[1], block[2], lds_bytes, stream,
                                       nullptr, extra);
   if (e != 0) return hip_fail("hipModuleLaunchKernel", e);
   return FRNN_OK;
@@ -312,6 +496,7 @@ int frnn_module_free(frnn_module_t m) {
   HipApi& h = hip();
   hipError_t e = 0;
   if (h.ok && m->mod) e = h.ModuleUnload(m->mod);
+  for (frnn_kernel_s* k : m->kernels) delete k;
   delete m;
   if (e != 0) return hip_fail("hipModuleUnload", e);
   return FRNN_OK;

@@ -51,10 +51,6 @@ template <int CTRL> __device__ __forceinline__ float dpp_mov(float x) {
 // x + (x of the lane 16 / 32 away): the gfx950 row swaps exchange the odd 16-lane rows of one
 // register with the even rows of another (the 32-lane halves for permlane32), so a register and
 // its copy come back as "own rows twice" and "partner rows twice"; no trip through LDS.
-#ifdef FRNN_HOST_HARNESS      // (the CPU test harness emulates lanes and has no such instruction)
-__device__ __forceinline__ float xor16_sum(float x) { return x + __shfl_xor(x, 16, 64); }
-__device__ __forceinline__ float xor32_sum(float x) { return x + __shfl_xor(x, 32, 64); }
-#else
 __device__ __forceinline__ float xor16_sum(float x) {
   const unsigned u = __builtin_bit_cast(unsigned, x);
   const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
@@ -65,7 +61,6 @@ __device__ __forceinline__ float xor32_sum(float x) {
   const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   return __builtin_bit_cast(float, (unsigned)r[0]) + __builtin_bit_cast(float, (unsigned)r[1]);
 }
-#endif
 template <int L> __device__ __forceinline__ float grp_allreduce(float x) {
   if constexpr (L >= 2) x += dpp_mov<0xB1>(x);    // quad_perm [1,0,3,2]
   if constexpr (L >= 4) x += dpp_mov<0x4E>(x);    // quad_perm [2,3,0,1]

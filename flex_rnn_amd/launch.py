@@ -12,6 +12,8 @@ from __future__ import annotations
 
 import contextlib
 import dataclasses
+import hashlib
+import json
 import os
 import struct
 import threading
@@ -198,6 +200,73 @@ def _fixed_picks() -> Dict[str, int]:
     return {k.strip(): int(v) for k, v in (kv.split('=') for kv in spec.split(',') if kv.strip())}
 
 
+class _Picks:
+    """The timed choice among the candidate builds of a kernel, kept per (kernel, candidate set, device,
+    batch, heads, rows) in memory and in `picks.json` beside the cached code objects, so that the choice -
+    and with it the order of the additions inside every reduction - is made once and then repeats: later
+    plans and later processes run the same build without timing anything.  The sequence length is not
+    part of the key: it changes how long a kernel runs, not which candidate is fastest, and calls over
+    pieces of a sequence then run the same code as one call over the whole."""
+
+    def __init__(self):
+        self.lock = threading.Lock()
+        self.mem: Dict[str, dict] = {}
+        self.loaded_from = None
+
+    @staticmethod
+    def key(name, builds, device_name, plan) -> str:
+        h = hashlib.sha256()
+        for spec, _, _ in builds:
+            h.update(runtime.source_key(spec.name, spec.source).encode())
+        return f'{name}|{h.hexdigest()[:20]}|{device_name}|B{plan.B}H{plan.H}M{plan.M}'
+
+    def _path(self):
+        return os.path.join(runtime.cache_dir(), 'picks.json')
+
+    def _load(self):
+        path = self._path()
+        if self.loaded_from != path:            # (the cache directory may be redirected between plans, e.g. by tests)
+            self.loaded_from = path
+            try:
+                with open(path) as f:
+                    disk = json.load(f)
+                for k, v in disk.items():
+                    self.mem.setdefault(k, v)
+            except (OSError, ValueError):
+                pass
+
+    def get(self, key, n):
+        with self.lock:
+            self._load()
+            rec = self.mem.get(key)
+        if rec and isinstance(rec.get('index'), int) and 0 <= rec['index'] < n:
+            return rec
+        return None
+
+    def put(self, key, index, times):
+        with self.lock:
+            self._load()
+            self.mem[key] = {'index': int(index), 'ms': [None if t == float('inf') else round(t, 5) for t in times]}
+            path = self._path()
+            try:                                # merge with what other processes wrote meanwhile; atomic replace
+                os.makedirs(os.path.dirname(path), exist_ok=True)
+                try:
+                    with open(path) as f:
+                        disk = json.load(f)
+                except (OSError, ValueError):
+                    disk = {}
+                disk.update(self.mem)
+                tmp = f'{path}.tmp{os.getpid()}_{threading.get_ident()}'
+                with open(tmp, 'w') as f:
+                    json.dump(disk, f, indent=0, sort_keys=True)
+                os.replace(tmp, path)
+            except OSError:
+                pass                            # a read-only cache: the choice still holds for this process
+
+
+PICKS = _Picks()
+
+
 class CompiledPlan:
     _tune_pending = frozenset()
 
@@ -264,6 +333,11 @@ class CompiledPlan:
         spec, kern, _ = self.builds[name][index]
         self.kernels[name] = (spec, kern)
         self._register(name, spec)
+        # the packed block must be exactly the argument segment the code object declares: a block that is
+        # short leaves the kernel reading pointers that were never set
+        declared = getattr(kern, 'arg_bytes', 0)
+        assert not declared or declared == self._packer[name].size, \
+            f'{name}: the host packs {self._packer[name].size} argument bytes, the code object declares {declared}'
 
     def _register(self, name, spec):
         pl = self.plan
@@ -321,8 +395,15 @@ class CompiledPlan:
         if name not in self._tune_pending or th.cuda.is_current_stream_capturing():
             return
         self._tune_pending.discard(name)
-        saved = [a.clone() for a in accumulators]
         n = len(self.builds[name])
+        dev = next(t.device for t in tensors.values() if t.is_cuda)
+        pkey = PICKS.key(name, self.builds[name], th.cuda.get_device_name(dev), self.plan)
+        rec = PICKS.get(pkey, n) if os.environ.get('FLEX_RNN_RETUNE', '0') == '0' else None
+        if rec is not None:                     # chosen before (by this or an earlier process): no timing
+            self._select(name, rec['index'])
+            self.build_times[name] = [float('inf') if t is None else t for t in rec.get('ms', [])] or None
+            return
+        saved = [a.clone() for a in accumulators]
         times = [float('inf')] * n
         usable = [True] * n
         # rounds over all candidates (the first untimed) rather than one candidate after the other: the
@@ -344,8 +425,10 @@ class CompiledPlan:
                     if i == 0:
                         raise                   # the first-ranked build must be launchable
                     usable[i] = False           # (a candidate the device refuses to launch is just not taken)
-        self._select(name, min(range(len(times)), key=times.__getitem__))
+        best = min(range(len(times)), key=times.__getitem__)
+        self._select(name, best)
         self.build_times[name] = times
+        PICKS.put(pkey, best, times)
         for a, s_ in zip(accumulators, saved):
             a.copy_(s_)
 

@@ -22,7 +22,28 @@ ARCH = 'gfx950'
 # (the resource-usage remarks land in the compile log; `kernel_resources` reads them back)
 EMITTER_OPTS = '-ffp-contract=fast -munsafe-fp-atomics -Rpass-analysis=kernel-resource-usage'
 
+# flags `frnn_compile` always passes (flex_rnn_amd/csrc/frnn_rt.cpp); part of the cache key, like the compiler's version
+FIXED_FLAGS = '--genco -O3 -std=c++17 -Xclang -target-feature -Xclang -packed-fp32-ops'
+
 _lib = None
+_toolchain = None
+
+
+def toolchain_id() -> str:
+    """What identifies the compiler behind `frnn_compile` (the version lines of `hipcc --version`): a code
+    object built by another compiler release must not be taken from the cache."""
+    global _toolchain
+    if _toolchain is None:
+        hipcc = os.environ.get('FRNN_HIPCC') or next(
+            (p for p in (os.path.join(os.environ.get('ROCM_PATH', '/opt/rocm'), 'bin', 'hipcc'), '/opt/rocm/bin/hipcc')
+             if os.access(p, os.X_OK)), 'hipcc')
+        try:
+            out = subprocess.run([hipcc, '--version'], capture_output=True, text=True, timeout=60).stdout
+            lines = [ln.strip() for ln in out.splitlines() if ln.startswith('HIP version') or 'clang version' in ln]
+            _toolchain = ' | '.join(lines) or 'unknown'
+        except (OSError, subprocess.SubprocessError):
+            _toolchain = 'unknown'
+    return _toolchain
 
 
 class RuntimeError_(RuntimeError):
@@ -34,7 +55,7 @@ def build_library(verbose: bool = False) -> str:
     src = os.path.join(_HERE, 'csrc', 'frnn_rt.cpp')
     inc = os.path.join(_ROOT, 'include')
     tmp = LIB_PATH + f'.tmp{os.getpid()}'
-    cmd = ['g++', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall', '-I', inc, src, '-o', tmp, '-ldl', '-pthread']
+    cmd = ['g++', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall', '-I', inc, '-I', os.path.join(_HERE, 'csrc'), src, '-o', tmp, '-ldl', '-pthread']
     if verbose:
         print(' '.join(cmd))
     subprocess.run(cmd, check=True)
@@ -53,6 +74,11 @@ def lib() -> ctypes.CDLL:
             f'{LIB_PATH} is missing: the HIP kernel runtime has not been built. '
             'Run `python -c "import __graft_entry__ as g; g.build()"` (or flex_rnn_amd.runtime.build_library()). '
             'There is no CPU fallback for the compiled path; use `.naive` for a pure-PyTorch run.')
+    try:
+        import torch  # noqa: F401  (its bundled HIP runtime must be in the process first: the library binds to the
+        #                            loaded copy by soname instead of bringing in a second one)
+    except ImportError:
+        pass
     L = ctypes.CDLL(LIB_PATH)
     L.frnn_version.restype = ctypes.c_int
     L.frnn_last_error.restype = ctypes.c_char_p
@@ -63,6 +89,8 @@ def lib() -> ctypes.CDLL:
     L.frnn_module_load.argtypes = [ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
     L.frnn_get_kernel.restype = ctypes.c_int
     L.frnn_get_kernel.argtypes = [ctypes.c_void_p, ctypes.c_char_p, ctypes.POINTER(ctypes.c_void_p)]
+    L.frnn_kernel_arg_bytes.restype = ctypes.c_int
+    L.frnn_kernel_arg_bytes.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_size_t)]
     L.frnn_launch.restype = ctypes.c_int
     L.frnn_launch.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
                               ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
@@ -74,7 +102,7 @@ def lib() -> ctypes.CDLL:
 
 
 EXPORTS = ('frnn_version', 'frnn_last_error', 'frnn_compile', 'frnn_module_load', 'frnn_get_kernel',
-           'frnn_launch', 'frnn_module_free', 'frnn_device_cus')
+           'frnn_kernel_arg_bytes', 'frnn_launch', 'frnn_module_free', 'frnn_device_cus')
 
 
 def _check(rc: int, what: str):
@@ -100,6 +128,10 @@ def cache_dir() -> str:
 def source_key(name: str, src: str, opts: str = EMITTER_OPTS) -> str:
     h = hashlib.sha256()
     h.update(ARCH.encode())
+    h.update(b'\0')
+    h.update(FIXED_FLAGS.encode())
+    h.update(b'\0')
+    h.update(toolchain_id().encode())
     h.update(b'\0')
     h.update(opts.encode())
     h.update(b'\0')
@@ -173,6 +205,9 @@ class Kernel:
         h = ctypes.c_void_p()
         _check(lib().frnn_get_kernel(module.handle, name.encode(), ctypes.byref(h)), f'looking up kernel {name}')
         self.handle = h
+        n = ctypes.c_size_t()
+        _check(lib().frnn_kernel_arg_bytes(h, ctypes.byref(n)), f'reading the argument size of kernel {name}')
+        self.arg_bytes = int(n.value)      # what the code object declares; 0 = unknown
 
     def launch(self, grid: Sequence[int], block: Sequence[int], args: bytes, stream: int = 0, lds_bytes: int = 0):
         g = _U3(*grid)

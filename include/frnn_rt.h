@@ -27,7 +27,7 @@ extern "C" {
 #endif
 
 typedef struct frnn_module_s* frnn_module_t;   /* opaque: a loaded code object            */
-typedef void* frnn_kernel_t;                   /* opaque: a kernel inside a loaded module */
+typedef struct frnn_kernel_s* frnn_kernel_t;   /* opaque: a kernel inside a loaded module */
 
 enum {
   FRNN_OK = 0,
@@ -63,11 +63,19 @@ int frnn_module_load(const char* path, frnn_module_t* out);
  * Replaces: getattr(torch.ops.<id>, func_name) (to_cuda.py:280). */
 int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out);
 
+/* Size in bytes of the kernel's argument segment as recorded in its code object (the
+ * `.kernarg_segment_size` of the AMDGPU metadata note), or 0 when the image carries no readable
+ * metadata.  `frnn_launch` rejects a block of any other size.
+ * Replaces: the typed C++ launcher the reference generates per kernel (to_cuda.py:236-247), where the
+ * compiler checks the argument list. */
+int frnn_kernel_arg_bytes(frnn_kernel_t k, size_t* out);
+
 /* Launch `k` with the given grid (in workgroups) and block (in threads) on `stream`
  * (a hipStream_t; NULL = default stream).  `args` points to `arg_bytes` bytes laid out
  * exactly as the kernel's parameter list (one by-value struct of 8-byte fields in this
- * project).  `arg_bytes` must equal the size of that parameter list and be a multiple of 8;
- * a shorter block would leave the kernel with unset arguments.  Returns after enqueueing;
+ * project).  `arg_bytes` must equal the size of that parameter list (checked against the code
+ * object's metadata, see frnn_kernel_arg_bytes) and be a multiple of 8; a shorter block would
+ * leave the kernel with unset arguments.  Returns after enqueueing;
  * stream-ordered, never synchronises.
  * Replaces: the generated `k<<<dim3(grid),dim3(threads)>>>(...)` launcher (to_cuda.py:245-247),
  * adding the stream and the error check the reference lacks. */

@@ -9,7 +9,6 @@
 // PROT_NONE guard page, so an out-of-bounds access ends the process with SIGSEGV instead of
 // passing silently.
 #pragma once
-#define FRNN_HOST_HARNESS 1
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -123,6 +122,27 @@ static inline int __builtin_amdgcn_update_dpp(int old, int src, int ctrl, int ro
 }
 
 static inline int __builtin_amdgcn_readfirstlane(int v) { return sim_lane_read(v, 0); }
+
+// gfx950 row swaps.  Both return the pair (new first operand, new second operand).
+// permlane16_swap exchanges the odd 16-lane rows of the first operand with the even rows of the
+// second: first' = [a.row0, b.row0, a.row2, b.row2], second' = [a.row1, b.row1, a.row3, b.row3].
+// permlane32_swap does the same with the 32-lane halves: first' = [a.lo, b.lo], second' = [a.hi, b.hi].
+struct sim_u2 {
+  unsigned v[2];
+  unsigned operator[](int i) const { return v[i]; }
+};
+static inline sim_u2 sim_permlane_swap(unsigned a, unsigned b, int width) {
+  const int lane = (int)threadIdx.x & 63;
+  const bool upper = (lane / width) & 1;                   // an odd row (the upper half)
+  const unsigned a_far = (unsigned)sim_lane_read((int)a, lane ^ width);
+  const unsigned b_far = (unsigned)sim_lane_read((int)b, lane ^ width);
+  sim_u2 r;
+  r.v[0] = upper ? b_far : a;       // odd rows of the first operand take the second operand's even rows
+  r.v[1] = upper ? b : a_far;       // even rows of the second operand take the first operand's odd rows
+  return r;
+}
+static inline sim_u2 __builtin_amdgcn_permlane16_swap(unsigned a, unsigned b, bool, bool) { return sim_permlane_swap(a, b, 16); }
+static inline sim_u2 __builtin_amdgcn_permlane32_swap(unsigned a, unsigned b, bool, bool) { return sim_permlane_swap(a, b, 32); }
 
 static inline float __shfl_xor(float v, int mask, int width = 64) {
   (void)width;

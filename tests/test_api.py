@@ -220,3 +220,30 @@ def test_row_kernel_candidate_tiles_are_valid():
                 t = dataclasses.replace(t, R1=r, W1=w) if reverse else dataclasses.replace(t, R=r, W=w)
                 planner.check_tile(t, plan.H, plan.NP, plan.part)
     assert (8, 16, 2, 8) in launch.row_kernel_tiles(prebuild.plan_for('rwkv7'), False)
+
+
+def test_timed_picks_are_kept_beside_the_cache(tmp_path, monkeypatch):
+    """The choice among candidate builds is stored per (kernel, candidates, device, B, H, M) - not per
+    sequence length - and found again by a fresh process (here: a fresh `_Picks`)."""
+    from flex_rnn_amd import launch, prebuild
+    from flex_rnn_amd.emit_hip import KernelSpec
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    builds = [(KernelSpec('frnn_fw', f'// candidate {i}', [], 64, ('1', '1', '1')), None, None) for i in range(3)]
+    long_plan = prebuild.plan_for('rwkv7', (2, 64, 2, 128, 128))
+    short_plan = prebuild.plan_for('rwkv7', (2, 32, 2, 128, 128))
+    other_plan = prebuild.plan_for('rwkv7', (4, 64, 2, 128, 128))
+    key = launch.PICKS.key('frnn_fw', builds, 'dev', long_plan)
+    assert key == launch.PICKS.key('frnn_fw', builds, 'dev', short_plan)
+    assert key != launch.PICKS.key('frnn_fw', builds, 'dev', other_plan)
+    assert key != launch.PICKS.key('frnn_fw', builds[:2], 'dev', long_plan)
+    assert key != launch.PICKS.key('frnn_fw', builds, 'other dev', long_plan)
+    a = launch._Picks()
+    assert a.get(key, 3) is None
+    a.put(key, 2, [0.5, float('inf'), 0.25])
+    assert a.get(key, 3)['index'] == 2
+    b = launch._Picks()                       # another process
+    rec = b.get(key, 3)
+    assert rec['index'] == 2 and rec['ms'] == [0.5, None, 0.25]
+    assert b.get(key, 2) is None              # a stored index that the candidate list no longer has is ignored
+    b.put('other', 0, [1.0])
+    assert launch._Picks().get(key, 3)['index'] == 2 and launch._Picks().get('other', 1)['index'] == 0

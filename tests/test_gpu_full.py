@@ -74,7 +74,9 @@ def test_chunked_call_equals_single_call_at_full_size():
     y1, S1 = g(*[x[:, :T // 2] for x in xs], *ss)
     h = flex_rnn_amd.jit(wl.step)
     y2, S2 = h(*[x[:, T // 2:] for x in xs], S1)
-    assert recurrence.rel_err(y1, y[:, :T // 2]) < 1e-3      # (equal unless the first-call timing picked other tiles)
+    # the same build of the forward kernel runs for both lengths (the timed choice is kept per batch, heads and
+    # rows, not per sequence length) and the forward pass accumulates nothing atomically: bit for bit
+    assert th.equal(y1, y[:, :T // 2])
     # the hand-off state passes through bf16 storage once more than inside a single call
     assert recurrence.rel_err(y2, y[:, T // 2:]) < 1e-2
     assert recurrence.rel_err(S2, S) < 1e-2

@@ -112,3 +112,72 @@ def test_launch_marshalling_against_stand_in_hip(runtime_lib, tmp_path):
     ''')
     r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
     assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr
+
+
+def test_argument_block_is_checked_against_the_code_object(runtime_lib, tmp_path, monkeypatch):
+    """`frnn_get_kernel` reads the kernel's argument-segment size from the code object's metadata note;
+    `frnn_launch` rejects a block of any other size (a block that is short would leave the kernel with
+    unset pointers), and the host refuses to register a kernel whose packed block has another size."""
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    src = ('#include <hip/hip_runtime.h>\nstruct TArg { void* p; long long s[5]; };\n'
+           'struct Args { TArg t[3]; long long B, T, H, M, nch; };\n'
+           'extern "C" __global__ void one(Args A) { ((float*)A.t[0].p)[threadIdx.x] = (float)A.B; }\n'
+           'extern "C" __global__ void two(float* p, int n, double x) { if ((int)threadIdx.x < n) p[threadIdx.x] = (float)x; }\n')
+    path = runtime.compile_kernel('pair', src)
+    so = tmp_path / 'libfakehip.so'
+    subprocess.run(['g++', '-shared', '-fPIC', '-o', str(so), os.path.join(ROOT, 'tests', 'fakehip', 'fakehip.cpp')], check=True)
+    code = textwrap.dedent(f'''
+        import ctypes, struct, sys
+        sys.path.insert(0, {ROOT!r})
+        fake = ctypes.CDLL({str(so)!r}, mode=ctypes.RTLD_GLOBAL)
+        from flex_rnn_amd import runtime
+        m = runtime.Module({path!r})
+        one, two = m.kernel('one'), m.kernel('two')
+        assert one.arg_bytes == 3 * 48 + 40, one.arg_bytes
+        assert two.arg_bytes == 24, two.arg_bytes
+        assert m.kernel('absent_from_metadata').arg_bytes == 0        # (the stand-in resolves any name)
+        good = bytes(3 * 48 + 40)
+        one.launch((1, 1, 1), (64, 1, 1), good)
+        for bad in (good[:-8], good + bytes(8), good[:48]):
+            try:
+                one.launch((1, 1, 1), (64, 1, 1), bad)
+            except RuntimeError as e:
+                assert 'declares 184' in str(e), e
+            else:
+                raise SystemExit('accepted a block of %d bytes' % len(bad))
+        # the host side: a plan whose packer disagrees with the code object is refused before any launch
+        from flex_rnn_amd.launch import CompiledPlan
+        from flex_rnn_amd.emit_hip import KernelSpec
+        class P: B = T = H = M = nchunks = 1
+        cp = CompiledPlan.__new__(CompiledPlan)
+        cp.plan, cp.kernels, cp._grid, cp._packer = P, {{}}, {{}}, {{}}
+        cp.builds = {{'one': [(KernelSpec('one', '', ['a', 'b', 'c'], 64, ('1', '1', '1')), one, None)],
+                     'short': [(KernelSpec('one', '', ['a', 'b'], 64, ('1', '1', '1')), one, None)]}}
+        cp._select('one', 0)
+        try:
+            cp._select('short', 0)
+        except AssertionError as e:
+            assert 'declares 184' in str(e), e
+        else:
+            raise SystemExit('registered a mis-sized argument block')
+        print('ok')
+    ''')
+    r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
+    assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr
+
+
+def test_cache_key_covers_fixed_flags_and_compiler(monkeypatch):
+    """The key of a cached code object changes with the source, the options, the flags the runtime always
+    passes (which must be the ones named in the C++ source) and the compiler's version."""
+    cpp = open(os.path.join(ROOT, 'flex_rnn_amd', 'csrc', 'frnn_rt.cpp')).read()
+    for flag in runtime.FIXED_FLAGS.split():
+        assert f'"{flag}"' in cpp, flag
+    assert 'version' in runtime.toolchain_id()
+    base = runtime.source_key('k', 'src')
+    assert base == runtime.source_key('k', 'src') and base != runtime.source_key('k', 'src2')
+    assert base != runtime.source_key('k', 'src', opts='-O1')
+    monkeypatch.setattr(runtime, 'FIXED_FLAGS', runtime.FIXED_FLAGS + ' -g')
+    assert runtime.source_key('k', 'src') != base
+    monkeypatch.undo()
+    monkeypatch.setattr(runtime, '_toolchain', 'HIP version: 0.0 | clang version 0')
+    assert runtime.source_key('k', 'src') != base
