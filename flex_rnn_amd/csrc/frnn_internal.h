@@ -6,7 +6,7 @@
 
 struct frnn_kernel_s {
   void* fn;            // hipFunction_t
-  size_t kernarg;      // size of the kernel's argument segment as its code object declares it (0 = unknown)
+  size_t kernarg;      // bytes of the kernel's explicit arguments as its code object declares them (0 = unknown)
 };
 
 // records the calling thread's error message (what frnn_last_error() returns) and returns `code`

@@ -246,7 +246,9 @@ struct MsgPack {
 
 bool key_is(const char* s, size_t n, const char* lit) { return n == strlen(lit) && memcmp(s, lit, n) == 0; }
 
-// kernarg segment size of `kernel` from an AMDGPU metadata blob; 0 when not found
+// Bytes of the explicit arguments of `kernel` (the end of its last argument that is not one of the
+// hidden ones the runtime appends, e.g. the grid size) from an AMDGPU metadata blob; 0 when not found.
+// Falls back to the whole argument segment for a kernel whose metadata lists no arguments.
 size_t kernarg_from_metadata(const uint8_t* d, size_t len, const char* kernel) {
   MsgPack m{d, d + len};
   size_t n;
@@ -260,8 +262,8 @@ size_t kernarg_from_metadata(const uint8_t* d, size_t len, const char* kernel) {
     for (size_t j = 0; j < nk && m.ok; j++) {
       size_t nf;
       if (!m.map(&nf)) return 0;
-      bool mine = false;
-      uint64_t size = 0;
+      bool mine = false, has_args = false;
+      uint64_t segment = 0, explicit_end = 0;
       for (size_t f = 0; f < nf && m.ok; f++) {
         const char* fk; size_t fkn;
         if (!m.str(&fk, &fkn)) return 0;
@@ -270,12 +272,34 @@ size_t kernarg_from_metadata(const uint8_t* d, size_t len, const char* kernel) {
           if (!m.str(&v, &vn)) return 0;
           mine = key_is(v, vn, kernel);
         } else if (key_is(fk, fkn, ".kernarg_segment_size")) {
-          if (!m.uint_(&size)) return 0;
+          if (!m.uint_(&segment)) return 0;
+        } else if (key_is(fk, fkn, ".args")) {
+          size_t na;
+          if (!m.array(&na)) return 0;
+          has_args = true;
+          for (size_t a = 0; a < na && m.ok; a++) {
+            size_t nq;
+            if (!m.map(&nq)) return 0;
+            uint64_t off = 0, size = 0;
+            bool hidden = false;
+            for (size_t q = 0; q < nq && m.ok; q++) {
+              const char* ak; size_t akn;
+              if (!m.str(&ak, &akn)) return 0;
+              if (key_is(ak, akn, ".offset")) { if (!m.uint_(&off)) return 0; }
+              else if (key_is(ak, akn, ".size")) { if (!m.uint_(&size)) return 0; }
+              else if (key_is(ak, akn, ".value_kind")) {
+                const char* v; size_t vn;
+                if (!m.str(&v, &vn)) return 0;
+                hidden = vn >= 7 && memcmp(v, "hidden_", 7) == 0;
+              } else m.skip();
+            }
+            if (!hidden && off + size > explicit_end) explicit_end = off + size;
+          }
         } else {
           m.skip();
         }
       }
-      if (mine && m.ok) return (size_t)size;
+      if (mine && m.ok) return (size_t)(has_args ? ((explicit_end + 7) & ~(uint64_t)7) : segment);
     }
     return 0;
   }
@@ -306,7 +330,7 @@ bool find_device_elf(const std::vector<char>& image, const uint8_t** elf, size_t
 }
 
 // 0 when the image has no readable metadata for `kernel` (the launch check is then skipped)
-size_t kernarg_segment_size(const std::vector<char>& image, const char* kernel) {
+size_t explicit_arg_bytes(const std::vector<char>& image, const char* kernel) {
   const uint8_t* e; size_t n;
   if (!find_device_elf(image, &e, &n) || n < 64 || e[4] != 2 /*ELFCLASS64*/ || e[5] != 1 /*little endian*/) return 0;
   uint64_t shoff; uint16_t shentsize, shnum;
@@ -455,7 +479,7 @@ int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out) {
   void* fn = nullptr;
   hipError_t e = h.ModuleGetFunction(&fn, m->mod, name);
   if (e != 0) return hip_fail("hipModuleGetFunction", e);
-  frnn_kernel_s* k = new frnn_kernel_s{fn, kernarg_segment_size(m->image, name)};
+  frnn_kernel_s* k = new frnn_kernel_s{fn, explicit_arg_bytes(m->image, name)};
   m->kernels.push_back(k);
   *out = k;
   return FRNN_OK;

@@ -386,6 +386,51 @@ class CompiledPlan:
             else:
                 kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
 
+    # ------------------------------------------------------------------ hidden buffers in the library's scratch
+    def static_layout(self):
+        """Where the hidden buffers of one forward + backward call of this plan (state checkpoints, saved row
+        sums, d-state checkpoints, saved backward sums) go inside the runtime's static scratch buffer:
+        {tensor name: (byte offset, bytes)}, offsets multiples of 256, and the total.  Raises when the plan
+        needs more than the buffer holds."""
+        pl, p = self.plan, self.plan.part
+        ck = pl.B * pl.H * pl.nchunks * pl.M * pl.NP * 4
+        row = pl.B * pl.H * pl.T * pl.M * 4
+        sizes = [(f'sck{k}', ck) for k in range(p.nstates)] + [('aux', len(p.aux) * row)] \
+            + [(f'dck{k}', ck) for k in range(p.nstates)] + [('daux', len(p.daux) * row)]
+        layout, off = {}, 0
+        for name, n in sizes:
+            if n:
+                layout[name] = (off, n)
+                off += -(-n // 256) * 256
+        assert off <= runtime.STATIC_SCRATCH_BYTES, \
+            f'the hidden buffers of this plan take {off} bytes, the static scratch buffer holds {runtime.STATIC_SCRATCH_BYTES}'
+        return layout, off
+
+    def launch_static(self, kname: str, tensors: Dict[str, th.Tensor], layout, clear=()):
+        """`_launch` through the runtime's entry point that allocates nothing: tensors named in `layout`
+        are not passed by the caller but live in the library's static scratch buffer (their pointer fields
+        are filled in by the library; the kernels address hidden buffers without strides)."""
+        spec, kern = self.kernels[kname]
+        pl = self.plan
+        vals, slots = [], []
+        dev = None
+        for j, name in enumerate(spec.tensors):
+            if name in layout:
+                off, n = layout[name]
+                slots.append((48 * j, off, n, 1 if name in clear else 0))
+                vals.extend([0] * 6)
+                continue
+            t = tensors[name]
+            assert t.is_cuda and (dev is None or t.device == dev), 'all tensors must live on one GPU'
+            dev = t.device
+            vals.append(t.data_ptr())
+            vals.extend(_strides5(t))
+        if not spec.tensors:
+            vals = [0] * 6
+        buf = self._packer[kname].pack(*vals, pl.B, pl.T, pl.H, pl.M, pl.nchunks)
+        with th.cuda.device(dev):
+            kern.launch_static(self._grid[kname], (spec.block, 1, 1), buf, slots, stream=th.cuda.current_stream(dev).cuda_stream)
+
     def _tune(self, name, tensors, accumulators=()):
         """Times every candidate build of kernel `name` on the tensors of this call (one untimed
         run, then the fastest of three timed ones, in rounds over the candidates) and keeps the

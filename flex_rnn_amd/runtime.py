@@ -19,6 +19,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _ROOT = os.path.dirname(_HERE)
 LIB_PATH = os.path.join(_HERE, 'libfrnn_rt.so')
 ARCH = 'gfx950'
+STATIC_SCRATCH_BYTES = 64 << 20       # FRNN_STATIC_SCRATCH_BYTES of include/frnn_rt.h
 # (the resource-usage remarks land in the compile log; `kernel_resources` reads them back)
 EMITTER_OPTS = '-ffp-contract=fast -munsafe-fp-atomics -Rpass-analysis=kernel-resource-usage'
 
@@ -51,11 +52,15 @@ class RuntimeError_(RuntimeError):
 
 
 def build_library(verbose: bool = False) -> str:
-    """Compile flex_rnn_amd/csrc/frnn_rt.cpp -> flex_rnn_amd/libfrnn_rt.so."""
-    src = os.path.join(_HERE, 'csrc', 'frnn_rt.cpp')
+    """Compile flex_rnn_amd/csrc/{frnn_rt.cpp, frnn_static.hip} -> flex_rnn_amd/libfrnn_rt.so (hipcc, gfx950: the
+    second file holds device code, the static scratch buffer and its fill kernel)."""
+    srcs = [os.path.join(_HERE, 'csrc', 'frnn_rt.cpp'), os.path.join(_HERE, 'csrc', 'frnn_static.hip')]
     inc = os.path.join(_ROOT, 'include')
     tmp = LIB_PATH + f'.tmp{os.getpid()}'
-    cmd = ['g++', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall', '-I', inc, '-I', os.path.join(_HERE, 'csrc'), src, '-o', tmp, '-ldl', '-pthread']
+    hipcc = os.environ.get('FRNN_HIPCC') or '/opt/rocm/bin/hipcc'
+    cmd = [hipcc, f'--offload-arch={ARCH}', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall',
+           '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
+           '-I', inc, '-I', os.path.join(_HERE, 'csrc'), *srcs, '-o', tmp, '-ldl', '-pthread']
     if verbose:
         print(' '.join(cmd))
     subprocess.run(cmd, check=True)
@@ -94,6 +99,10 @@ def lib() -> ctypes.CDLL:
     L.frnn_launch.restype = ctypes.c_int
     L.frnn_launch.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
                               ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+    L.frnn_launch_static.restype = ctypes.c_int
+    L.frnn_launch_static.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32),
+                                     ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t,
+                                     ctypes.c_void_p, ctypes.c_size_t]
     L.frnn_module_free.restype = ctypes.c_int
     L.frnn_module_free.argtypes = [ctypes.c_void_p]
     L.frnn_device_cus.restype = ctypes.c_int
@@ -102,7 +111,7 @@ def lib() -> ctypes.CDLL:
 
 
 EXPORTS = ('frnn_version', 'frnn_last_error', 'frnn_compile', 'frnn_module_load', 'frnn_get_kernel',
-           'frnn_kernel_arg_bytes', 'frnn_launch', 'frnn_module_free', 'frnn_device_cus')
+           'frnn_kernel_arg_bytes', 'frnn_launch', 'frnn_launch_static', 'frnn_module_free', 'frnn_device_cus')
 
 
 def _check(rc: int, what: str):
@@ -214,6 +223,18 @@ class Kernel:
         b = _U3(*block)
         _check(lib().frnn_launch(self.handle, g, b, lds_bytes, ctypes.c_void_p(stream), args, len(args)),
                f'launching kernel {self.name}')
+
+
+    def launch_static(self, grid: Sequence[int], block: Sequence[int], args: bytes, slots, stream: int = 0, lds_bytes: int = 0):
+        """`launch` with the hidden buffers named by `slots` - (byte offset of the pointer field in `args`,
+        byte offset inside the library's static scratch buffer, size in bytes, clear first?) each - placed
+        in that buffer by the library; allocates nothing."""
+        g = _U3(*grid)
+        b = _U3(*block)
+        arr = (ctypes.c_uint64 * (4 * max(len(slots), 1)))(*[int(v) for s in slots for v in s])
+        _check(lib().frnn_launch_static(self.handle, g, b, lds_bytes, ctypes.c_void_p(stream), args, len(args),
+                                        ctypes.cast(arr, ctypes.c_void_p), len(slots)),
+               f'launching kernel {self.name} on the static scratch buffer')
 
 
 class Module:

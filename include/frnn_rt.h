@@ -63,9 +63,10 @@ int frnn_module_load(const char* path, frnn_module_t* out);
  * Replaces: getattr(torch.ops.<id>, func_name) (to_cuda.py:280). */
 int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out);
 
-/* Size in bytes of the kernel's argument segment as recorded in its code object (the
- * `.kernarg_segment_size` of the AMDGPU metadata note), or 0 when the image carries no readable
- * metadata.  `frnn_launch` rejects a block of any other size.
+/* Size in bytes of the kernel's explicit arguments as recorded in its code object (the `.args` of
+ * the AMDGPU metadata note up to the end of the last argument that is not a hidden one, rounded up
+ * to 8), or 0 when the image carries no readable metadata.  `frnn_launch` rejects a block of any
+ * other size.
  * Replaces: the typed C++ launcher the reference generates per kernel (to_cuda.py:236-247), where the
  * compiler checks the argument list. */
 int frnn_kernel_arg_bytes(frnn_kernel_t k, size_t* out);
@@ -81,6 +82,37 @@ int frnn_kernel_arg_bytes(frnn_kernel_t k, size_t* out);
  * adding the stream and the error check the reference lacks. */
 int frnn_launch(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3],
                 uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes);
+
+/* Size of the library's static scratch buffer, per GPU (see frnn_launch_static). */
+#define FRNN_STATIC_SCRATCH_BYTES (64ull << 20)
+
+/* One hidden buffer of a launch that is to live in the library's static scratch buffer. */
+typedef struct frnn_scratch_slot {
+  uint64_t arg_offset;     /* byte offset, in the argument block, of the 8-byte pointer field to fill in  */
+  uint64_t scratch_offset; /* where the region starts inside the scratch buffer; a multiple of 256         */
+  uint64_t bytes;          /* size of the region; offset + bytes <= FRNN_STATIC_SCRATCH_BYTES              */
+  uint64_t clear;          /* non-zero: the region is zero-filled on `stream` before the kernel runs       */
+} frnn_scratch_slot;
+
+/* frnn_launch for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose
+ * `forward` / `backward` allocate the checkpoints and saved sums with torch on every call
+ * (twopass.py:224-228, 349-356).  Same as frnn_launch, except that the pointer fields of `args`
+ * named by `slots` are filled in by the library with addresses inside a buffer of
+ * FRNN_STATIC_SCRATCH_BYTES that is part of the library's device image (every GPU the library runs on
+ * holds one until the process ends).  The caller chooses the layout (`scratch_offset`), so several
+ * launches can share regions: the forward kernel writes the checkpoints where the backward kernels
+ * of the same call read them.  Inputs and outputs are still passed by the caller.  The call
+ * allocates and frees nothing and never synchronises; regions marked `clear` are zeroed by a fill
+ * kernel on `stream` (no memset node, so the call may be captured into a graph).  A region that does
+ * not fit, is misaligned or overlaps another one of the same call is rejected with FRNN_ERR_ARG: use
+ * frnn_launch with caller-allocated buffers for such sizes.  The buffer keeps what the last launch
+ * left in it.  All calls on one GPU share it: calls whose kernels may overlap in time on one GPU
+ * (other streams, other threads) race unless their regions are disjoint.  The first call on each
+ * device looks the buffer's address up and must not be made during stream capture. */
+int frnn_launch_static(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3],
+                       uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
+                       const frnn_scratch_slot* slots, size_t nslots);
 
 /* Unload a module.  Kernels obtained from it become invalid. */
 int frnn_module_free(frnn_module_t m);

@@ -122,7 +122,9 @@ def test_argument_block_is_checked_against_the_code_object(runtime_lib, tmp_path
     src = ('#include <hip/hip_runtime.h>\nstruct TArg { void* p; long long s[5]; };\n'
            'struct Args { TArg t[3]; long long B, T, H, M, nch; };\n'
            'extern "C" __global__ void one(Args A) { ((float*)A.t[0].p)[threadIdx.x] = (float)A.B; }\n'
-           'extern "C" __global__ void two(float* p, int n, double x) { if ((int)threadIdx.x < n) p[threadIdx.x] = (float)x; }\n')
+           'extern "C" __global__ void two(float* p, int n, double x) { if ((int)threadIdx.x < n) p[threadIdx.x] = (float)x; }\n'
+           # (uses the grid size: the compiler appends hidden arguments, which the launcher fills in, not the caller)
+           'extern "C" __global__ void three(float* p, int n) { for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 1.0f; }\n')
     path = runtime.compile_kernel('pair', src)
     so = tmp_path / 'libfakehip.so'
     subprocess.run(['g++', '-shared', '-fPIC', '-o', str(so), os.path.join(ROOT, 'tests', 'fakehip', 'fakehip.cpp')], check=True)
@@ -135,6 +137,7 @@ def test_argument_block_is_checked_against_the_code_object(runtime_lib, tmp_path
         one, two = m.kernel('one'), m.kernel('two')
         assert one.arg_bytes == 3 * 48 + 40, one.arg_bytes
         assert two.arg_bytes == 24, two.arg_bytes
+        assert m.kernel('three').arg_bytes == 16
         assert m.kernel('absent_from_metadata').arg_bytes == 0        # (the stand-in resolves any name)
         good = bytes(3 * 48 + 40)
         one.launch((1, 1, 1), (64, 1, 1), good)
@@ -181,3 +184,43 @@ def test_cache_key_covers_fixed_flags_and_compiler(monkeypatch):
     monkeypatch.undo()
     monkeypatch.setattr(runtime, '_toolchain', 'HIP version: 0.0 | clang version 0')
     assert runtime.source_key('k', 'src') != base
+
+
+def test_static_scratch_launch_validates_before_touching_the_device(runtime_lib, tmp_path):
+    """`frnn_launch_static` refuses regions that do not fit its buffer, are misaligned, overlap or name a
+    pointer field outside the argument block - all before any device call, so this runs without a GPU."""
+    hdr = open(os.path.join(ROOT, 'include', 'frnn_rt.h')).read()
+    assert re.search(r'#define FRNN_STATIC_SCRATCH_BYTES \(64ull << 20\)', hdr) and runtime.STATIC_SCRATCH_BYTES == 64 << 20
+    so = tmp_path / 'libfakehip.so'
+    subprocess.run(['g++', '-shared', '-fPIC', '-o', str(so), os.path.join(ROOT, 'tests', 'fakehip', 'fakehip.cpp')], check=True)
+    code = textwrap.dedent(f'''
+        import ctypes, sys
+        sys.path.insert(0, {ROOT!r})
+        fake = ctypes.CDLL({str(so)!r}, mode=ctypes.RTLD_GLOBAL)
+        from flex_rnn_amd import runtime
+        open({str(so)!r} + '.img', 'wb').write(bytes([127]) + b'ELF' + bytes(100)); k = runtime.Module({str(so)!r} + '.img').kernel('x')
+        cap = runtime.STATIC_SCRATCH_BYTES
+        args = bytes(48)
+        cases = [([(0, 0, cap + 1, 0)], 'do not fit'), ([(0, cap, 256, 0)], 'do not fit'), ([(0, 256, 0, 0)], 'do not fit'),
+                 ([(0, 100, 256, 0)], 'multiple of 256'), ([(0, 0, 300, 0), (8, 256, 256, 0)], 'overlap'),
+                 ([(0, 0, 256, 0), (0, 256, 256, 0)], 'same pointer field'), ([(48, 0, 256, 0)], 'outside'),
+                 ([(12, 0, 256, 0)], 'misaligned'), ([(0, i * 256, 256, 0) for i in range(65)], 'at most 64')]
+        for slots, msg in cases:
+            try:
+                k.launch_static((1, 1, 1), (64, 1, 1), args, slots)
+            except RuntimeError as e:
+                assert msg in str(e), (msg, str(e))
+            else:
+                raise SystemExit('accepted ' + str(slots))
+        for kw, msg in [(dict(args=bytes(44)), 'multiple of 8'), (dict(args=bytes(8192)), 'at most 4096'), (dict(grid=(0, 1, 1)), 'empty grid')]:
+            a = dict(grid=(1, 1, 1), args=args); a.update(kw)
+            try:
+                k.launch_static(a['grid'], (64, 1, 1), a['args'], [])
+            except RuntimeError as e:
+                assert msg in str(e), (msg, str(e))
+            else:
+                raise SystemExit('accepted ' + str(kw))
+        print('ok')
+    ''')
+    r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
+    assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr
