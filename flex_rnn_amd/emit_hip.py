@@ -493,6 +493,12 @@ class Emitter:
                 f'#define COLC(c) {f"(min(COL(c), {self.N - 1}))" if self.pad else "COL(c)"}\n'
                 '#define ROWC(r) (min(row0 + (r), M - 1))\n')
 
+    def _row_attr(self) -> str:
+        """Occupancy request of the row kernels (`TileConfig.WPE` waves per SIMD): the compiler then fits the
+        kernel into 512 / WPE registers instead of using all a workgroup of its size may have."""
+        wpe = int(getattr(self.tile, 'WPE', 0) or 0)
+        return f' __attribute__((amdgpu_waves_per_eu({wpe},{wpe})))' if wpe else ''
+
     def _lane_prolog(self) -> str:
         """What a device function needs to evaluate COL(c) on its own (only emitted with padding)."""
         return f'const int l = (threadIdx.x & 63) % {self.tile.L};' if self.pad else ''
@@ -510,18 +516,52 @@ class Emitter:
         else:
             st.add(f's_in{i}', 1, dt, A.p(f'in{i}'), lambda tt, x, i=i: self._in_index(A, i, t=tt), ts)
 
-    def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str) -> str:
+    @staticmethod
+    def _operand_order(g: Graph, names, skip=()):
+        """(early, order): `early` = those of the graph inputs `names` that the first row sum of `g` depends on
+        (a step cannot start before it has them), `order` = all of `names`, the early ones first, the rest by
+        first use.  States (`skip`) are registers, not LDS operands."""
+        nm = g.node_map()
+        first = next((n for n in g.nodes if n.op == 'sum'), None)
+        seen = set()
+        if first is not None:
+            stack = [first.name]
+            while stack:
+                v = stack.pop()
+                if v not in seen:
+                    seen.add(v)
+                    if v in nm:
+                        stack.extend(nm[v].value_args())
+        early = [v for v in names if v in seen and v not in skip]
+        pos = {}
+        for k, n in enumerate(g.nodes):
+            for a in n.value_args():
+                pos.setdefault(a, k)
+        rest = sorted((v for v in names if v not in early), key=lambda v: pos.get(v, len(g.nodes)))
+        return early, early + rest
+
+    def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str, decl: bool = True) -> str:
         """Registers <- staged LDS operand for timestep tt."""
         rr, cc = _dims(ext, R, C)
         if ext == (False, True):
-            return (f'      float {var}[1][{C}];\n#pragma unroll\n      for (int c = 0; c < {C}; c++) '
+            return ((f'      float {var}[1][{C}];\n' if decl else '') + f'#pragma unroll\n      for (int c = 0; c < {C}; c++) '
                     f'{var}[0][c] = {sname}[{tt}][COL(c)];\n')
         if ext == (True, False):
-            return (f'      float {var}[{R}][1];\n#pragma unroll\n      for (int r = 0; r < {R}; r++) '
+            return ((f'      float {var}[{R}][1];\n' if decl else '') + f'#pragma unroll\n      for (int r = 0; r < {R}; r++) '
                     f'{var}[r][0] = {sname}[{tt}][rloc + r];\n')
         if ext == (False, False):
-            return f'      float {var}[1][1]; {var}[0][0] = {sname}[{tt}][0];\n'
+            return (f'      float {var}[1][1]; ' if decl else '      ') + f'{var}[0][0] = {sname}[{tt}][0];\n'
         raise AssertionError
+
+    def _ahead_operand(self, var: str, sname: str, ext, R: int, C: int, nxt: str):
+        """An operand that is read from LDS one step ahead.  Returns (code before the time loop: the first
+        step's value into `<var>n`; code inside the loop: this step's value out of `<var>n` into `var`, and the
+        next step's - staged timestep `nxt`, clamped to the staged range by the caller - into `<var>n`)."""
+        rr, cc = _dims(ext, R, C)
+        copy = (f'      float {var}[{rr}][{cc}];\n#pragma unroll\n      for (int r = 0; r < {rr}; r++)\n#pragma unroll\n'
+                f'      for (int c = 0; c < {cc}; c++) {var}[r][c] = {var}n[r][c];\n')
+        return (lambda first: self._load_operand(f'{var}n', sname, ext, R, C, first),
+                copy + self._load_operand(f'{var}n', sname, ext, R, C, nxt, decl=False))
 
     def _load_const_input(self, A: _Args, i: int, R: int, C: int) -> str:
         """Time-independent input -> registers, once."""
@@ -609,20 +649,31 @@ class Emitter:
         body.append('    __syncthreads();\n')
         body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
-        body.append(f'#pragma unroll 2\n    for (int tt = 0; tt < nt; tt++) {{\n')
+        # LDS operands of a step, in the order the step needs them; those its first row sum depends on are read one
+        # step ahead (the sum, and with it everything else of the step, would otherwise wait for the LDS)
+        operands = {}                       # graph input -> (register array, LDS array, extent)
+        for nm_ in used:
+            if nm_ in p.in_names and self.tdep[p.in_names.index(nm_)]:
+                i = p.in_names.index(nm_)
+                operands[nm_] = (f'x{i}', f's_in{i}', self.in_ext(i))
+            elif nm_ in rfront:
+                operands[nm_] = (f'd{rfront.index(nm_)}', f's_d{rfront.index(nm_)}', (False, True))
+        early, order = self._operand_order(g, list(operands), skip=p.st_names)
+        early = {0: [], 1: early}.get(getattr(t, 'PF', 1), order)          # (PF = 2: every operand a step ahead)
+        ahead = {nm_: self._ahead_operand(*operands[nm_], R, C, f'min(tt + 1, {TS - 1})') for nm_ in early}
+        for nm_ in early:
+            body.append(ahead[nm_][0]('0'))
+        body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = 0; tt < nt; tt++) {{\n')
+        for nm_ in order:
+            body.append(ahead[nm_][1] if nm_ in ahead else self._load_operand(*operands[nm_], R, C, 'tt'))
         call = []
         for nm_ in used:
             if nm_ in p.in_names:
-                i = p.in_names.index(nm_)
-                if self.tdep[i]:
-                    body.append(self._load_operand(f'x{i}', f's_in{i}', self.in_ext(i), R, C, 'tt'))
-                call.append(f'x{i}')
+                call.append(f'x{p.in_names.index(nm_)}')
             elif nm_ in p.st_names:
                 call.append(f'S{p.st_names.index(nm_)}')
             elif nm_ in rfront:
-                q = rfront.index(nm_)
-                body.append(self._load_operand(f'd{q}', f's_d{q}', (False, True), R, C, 'tt'))
-                call.append(f'd{q}')
+                call.append(f'd{rfront.index(nm_)}')
             else:
                 raise AssertionError(nm_)
         rrs = R if st_ext[0][0] else 1
@@ -640,7 +691,10 @@ class Emitter:
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
             body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++)\n#pragma unroll\n      for (int c = 0; c < {cc}; c++) S{k}[r][c] = nS{k}[r][c];\n')
-        body.append('      if (l == 0) {\n')
+        # every lane of a group holds the row sums after the all-reduce and stores them (same address, same value):
+        # a store by one lane only would put a branch into every timestep and keep the compiler from overlapping
+        # the next step's LDS reads and state-independent arithmetic with this step
+        body.append('      {\n' if getattr(t, 'NB', 1) & 1 else '      if (l == 0) {\n')
         for k in range(nout):
             body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_out{k}[tt][rloc + r] = y{k}[{"r" if rrs > 1 else "0"}][0];\n')
         for k in range(naux):
@@ -664,7 +718,7 @@ class Emitter:
             body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) {self._col_if()}stf<{dt}>({A.p(nm)}, '
                         f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, S{k}[r][c]); }}\n')
-        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) {kname}(Args A) {{\n'
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){self._row_attr()} {kname}(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
         source = PRELUDE + A.struct() + self._row_macros() + fn_src + '\n' + kernel
         return KernelSpec(kname, source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
@@ -783,16 +837,19 @@ class Emitter:
         shared_in = [i for i in used_in if needs_state and self.tdep[i] and not self.in_ext(i)[1]
                      and p.in_names[i] in used and p.in_names[i] in re_used]
 
-        def operand_loads(tt, names, state_var):
-            code, call = [], []
+        def operand_loads(tt, names, state_var, ahead=None, order=None):
+            """Loads of the LDS operands among `names` for timestep `tt` and the argument list.  With `order` the
+            loads come in that order; those in `ahead` were read one step earlier (see `_ahead_operand`)."""
+            code, call, loads = [], [], {}
             for nm_ in names:
                 if nm_ in p.in_names:
                     i = p.in_names.index(nm_)
                     if i in shared_in:
                         call.append(f'x{i}_{tt}')
                     elif self.tdep[i]:
-                        code.append(self._load_operand(f'x{i}_{tt}' if needs_state else f'x{i}', f's_in{i}', self.in_ext(i), R, C, tt))
-                        call.append(f'x{i}_{tt}' if needs_state else f'x{i}')
+                        v = f'x{i}_{tt}' if needs_state else f'x{i}'
+                        loads[nm_] = (v, f's_in{i}', self.in_ext(i))
+                        call.append(v)
                     else:
                         call.append(f'x{i}')
                 elif nm_ in p.st_names:
@@ -801,26 +858,29 @@ class Emitter:
                     k = p.aux.index(nm_)
                     e = self.jext[nm_]
                     v = f'ax{k}_{tt}' if needs_state else f'ax{k}'
-                    code.append(self._load_operand(v, f's_aux{k}', (e[0], False), R, C, tt))
+                    loads[nm_] = (v, f's_aux{k}', (e[0], False))
                     call.append(v)
                 elif nm_ in p.dout_names:
                     k = p.dout_names.index(nm_)
                     v = f'dy{k}_{tt}' if needs_state else f'dy{k}'
-                    code.append(self._load_operand(v, f's_dy{k}', colx, R, C, tt))
+                    loads[nm_] = (v, f's_dy{k}', colx)
                     call.append(v)
                 elif nm_ in p.dnst_names:
                     call.append(f'D{p.dnst_names.index(nm_)}')
                 elif nm_ in rfront:
                     q = rfront.index(nm_)
                     v = f'd{q}_{tt}' if needs_state else f'd{q}'
-                    code.append(self._load_operand(v, f's_d{q}', (False, True), R, C, tt))
+                    loads[nm_] = (v, f's_d{q}', (False, True))
                     call.append(v)
                 else:
                     raise AssertionError(nm_)
-            return code, call
+            for nm_ in (order if order is not None else list(loads)):
+                if nm_ in loads:
+                    code.append(ahead[nm_][1] if ahead and nm_ in ahead else self._load_operand(*loads[nm_], R, C, tt))
+            return code, call, loads
 
-        def dstep_block(tt, state_var, indent='      '):
-            code, call = operand_loads(tt, used, state_var)
+        def dstep_block(tt, state_var, indent='      ', ahead=None, order=None):
+            code, call, _ = operand_loads(tt, used, state_var, ahead, order)
             for k in range(nst):
                 rr, cc = _dims(st_ext[k], R, C)
                 code.append(f'{indent}float nD{k}[{rr}][{cc}];\n')
@@ -842,7 +902,8 @@ class Emitter:
                 code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {rr}; r++)\n#pragma unroll\n{indent}for (int c = 0; c < {cc}; c++) D{k}[r][c] = nD{k}[r][c];\n')
             for i in const_col:
                 code.append(f'#pragma unroll\n{indent}for (int r = 0; r < {rrs}; r++) gacc{i}[r][0] += gc{i}[r][0];\n')
-            code.append(f'{indent}if (l == 0) {{\n')
+            # (as in the forward kernel: with bit 1 of NB all lanes of a group store the same sums, no branch inside the time loop)
+            code.append(f'{indent}{{\n' if getattr(t, 'NB', 1) & 2 else f'{indent}if (l == 0) {{\n')
             ridx = 'r' if rrs > 1 else '0'
             for i in tdep_col:
                 code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_dc{i}[{tt}][rloc + r] = gc{i}[{ridx}][0];\n')
@@ -852,8 +913,16 @@ class Emitter:
             return code
 
         if not needs_state:
-            body.append(f'#pragma unroll 2\n    for (int tt = nt - 1; tt >= 0; tt--) {{\n')
-            body += dstep_block('tt', lambda k: (_ for _ in ()).throw(AssertionError()))
+            # operands in the order the step needs them; those of its first row sum are read one step ahead
+            no_state = lambda k: (_ for _ in ()).throw(AssertionError())
+            _, _, loads = operand_loads('tt', used, no_state)
+            early, order = self._operand_order(g, list(loads), skip=p.dnst_names)
+            early = {0: [], 1: early}.get(getattr(t, 'PF', 1), order)      # (PF = 2: every operand a step ahead)
+            ahead = {nm_: self._ahead_operand(*loads[nm_], R, C, 'max(tt - 1, 0)') for nm_ in early}
+            for nm_ in early:
+                body.append(ahead[nm_][0]('nt - 1'))
+            body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = nt - 1; tt >= 0; tt--) {{\n')
+            body += dstep_block('tt', no_state, ahead=ahead, order=order)
             body.append('    }\n')
         else:
             # recompute the DT states of this chunk from its checkpoint, then walk back
@@ -866,7 +935,7 @@ class Emitter:
                     body.append(self._load_operand(f'x{i}_{tt}', f's_in{i}', self.in_ext(i), R, C, str(tt)))
             for tt in range(DT - 1):
                 body.append(f'    if ({tt + 1} < nt) {{\n' if tail else '    {\n')
-                code, call = operand_loads(str(tt), re_used, lambda k, tt=tt: f'Sh{k}_{tt}')
+                code, call, _ = operand_loads(str(tt), re_used, lambda k, tt=tt: f'Sh{k}_{tt}')
                 body += code
                 for k in range(nst):
                     call.append(f'Sh{k}_{tt + 1}')
@@ -911,7 +980,7 @@ class Emitter:
             body.append(f'#pragma unroll\n  for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
                         f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) {self._col_if()}stf<{dt}>({A.p(nm)}, '
                         f'(i64)b * {A.s(nm, 0)} + (i64)h * {A.s(nm, 1)} + (i64)(row0 + r) * {A.s(nm, 2)} + (i64)COL(c) * {A.s(nm, 3)}, D{k}[r][c]); }}\n')
-        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}) frnn_bw1(Args A) {{\n'
+        kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){self._row_attr()} frnn_bw1(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
         source = PRELUDE + A.struct() + self._row_macros() + '\n'.join(fns) + '\n' + kernel
         return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
@@ -1008,14 +1077,34 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   }}
 }}
 '''
+        helper += '''
+// x summed over the 64 / N_ instances of a wave (lanes N_ apart); every lane gets the total
+template <int N_> __device__ __forceinline__ float inst_total(float x) {
+  if constexpr (N_ <= 16) x = xor16_sum(x);
+  if constexpr (N_ <= 32) x = xor32_sum(x);
+  return x;
+}
+'''
         b = []
-        rows_decl = ('  const int mlo = 0, mhi = M;' if MS == 1 else
-                     f'  const int mlo = blockIdx.z * {MR}, mhi = min(M, mlo + {MR});   // rows of this instance\n'
-                     '  if (mlo >= M) return;')
+        # Narrow states pack IPB = 64 / N instances into a wave.  With split rows they are IPB consecutive row slices
+        # of one chunk (`share`): the wave then reads whole 128-byte lines of every per-row operand (a slice of 16 fp32
+        # rows is half a line; with the instances on different chunks every line was fetched twice), and the slices'
+        # row / scalar gradients - which meet in the same addresses - are summed across the wave's instances with
+        # lane swaps before one instance adds them to memory.  Otherwise the instances of a wave are IPB chunks.
+        share = IPB > 1 and MS > 1 and MS % IPB == 0 and N in (16, 32) and HB == 1
+        if MS == 1:
+            rows_decl = '  const int mlo = 0, mhi = M;'
+        elif share:
+            rows_decl = (f'  const int mlo = (blockIdx.z * {IPB} + inst) * {MR}, mhi = min(M, mlo + {MR});   // rows of this instance\n'
+                         '  valid = valid && mlo < M;               // (a slice beyond the last row walks no rows and adds nothing)')
+        else:
+            rows_decl = (f'  const int mlo = blockIdx.z * {MR}, mhi = min(M, mlo + {MR});   // rows of this instance\n'
+                         '  if (mlo >= M) return;')
+        cpb = 1 if share else IPB           # chunks per workgroup
         # grid y is limited to 65535 blocks: with more (batch, head group) pairs than that, both indices
         # travel in x, in the same order of dispatch
         fold = plan.B * (plan.H // HB) > MAX_GRID_Y
-        block_decl = (f'  const int gx_ = (nch + {IPB - 1}) / {IPB};\n  const int bx_ = blockIdx.x % gx_, by_ = blockIdx.x / gx_;\n'
+        block_decl = (f'  const int gx_ = (nch + {cpb - 1}) / {cpb};\n  const int bx_ = blockIdx.x % gx_, by_ = blockIdx.x / gx_;\n'
                       if fold else '')
         bx, by = ('bx_', 'by_') if fold else ('blockIdx.x', 'blockIdx.y')
         b.append(f'''  const int tid = threadIdx.x;
@@ -1025,8 +1114,8 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
   const int inst = {"tid / " + str(N) if IPB > 1 else "0"};
   const int T = (int)A.T, H = (int)A.H, M = (int)A.M, nch = (int)A.nch;
   (void)T;
-{block_decl}  int ch = {bx} * {IPB} + inst;
-  const bool valid = ch < nch;
+{block_decl}  int ch = {f"{bx}" if share else f"{bx} * {IPB} + inst"};
+  bool valid = ch < nch;
   if (!valid) ch = nch - 1;
   const int HG = H / {HB};                     // head groups; an instance walks {HB} heads
   const int b = {by} / HG, h0 = ({by} % HG) * {HB};
@@ -1176,7 +1265,10 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             b.append(f'  const float* dckp{k} = (const float*){A.p(f"dck{k}")} + (((i64)bh * nch + ch) * M) * {N} + n;\n')
             for j in range(PDe):
                 b.append(f'  float Sq{k}_{j} = sckp{k}[min(mlo + {j}, M - 1) * {N}];\n  float Dq{k}_{j} = dckp{k}[min(mlo + {j}, M - 1) * {N}];\n')
-        b.append(f'  for (int m0 = mlo; m0 < mhi; m0 += {MB}) {{\n')
+        if share:       # (the same number of row blocks for every instance of the wave: there are barriers inside)
+            b.append(f'  for (int mi_ = 0; mi_ < {MR}; mi_ += {MB}) {{ const int m0 = mlo + mi_;\n')
+        else:
+            b.append(f'  for (int m0 = mlo; m0 < mhi; m0 += {MB}) {{\n')
         if rowops:
             b.append('    __syncthreads();\n')
             # fixed trip count, fully unrolled: every load of the block is in flight before the
@@ -1304,11 +1396,13 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
             nmv = f'din{i}'
             ext = self.in_ext(i)
             bB, bT, bH = bflags(i)
-            cond = 'valid' + ((' && nok' if self.pad else '') if ext[1] else ' && n == 0')
+            cond = ('inst == 0' if share else 'valid') + ((' && nok' if self.pad else '') if ext[1] else ' && n == 0')
             if tail and not bT:
                 cond += f' && t0 + {tt} < T'
             idx = out_index(i, tt, hexpr)
             if bB or bT or (bH and HB < plan.H) or MS > 1:
+                if share:       # the wave's instances hold slices of the same sum: all lanes add them up, one instance writes
+                    return f'{ind}{{ const float tot_ = inst_total<{N}>({val}); if ({cond}) atomic_addf({A.p(nmv)}, {idx}, tot_); }}\n'
                 return f'{ind}if ({cond}) atomic_addf({A.p(nmv)}, {idx}, {val});\n'
             dt = 0 if i in self.atomic else DT_CODE[plan.in_dtypes[i]]      # broadcast inputs use fp32 scratch
             return f'{ind}if ({cond}) stf<{dt}>({A.p(nmv)}, {idx}, {val});\n'
@@ -1377,5 +1471,5 @@ template <int N_> __device__ __forceinline__ float inst_allreduce(float x) {{
         attr = f' __attribute__((amdgpu_waves_per_eu({wpe},{wpe})))' if wpe else ''
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){attr} frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
         source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + pre_src + '\n' + kernel
-        gx, gy = f'(nch + {IPB - 1}) // {IPB}', f'B * (H // {HB})'
-        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'({gx}) * {gy}', '1', str(MS)) if fold else (gx, gy, str(MS)))
+        gx, gy, gz = f'(nch + {cpb - 1}) // {cpb}', f'B * (H // {HB})', str(MS // IPB if share else MS)
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'({gx}) * {gy}', '1', gz) if fold else (gx, gy, gz))

@@ -159,15 +159,41 @@ def row_kernel_tiles(plan, reverse: bool):
     return out
 
 
-def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save: bool = True):
-    """[(spec, path)] for `row_kernel_tiles`, compiled side by side (`save=False`: the inference
-    variant of the forward kernel)."""
-    specs = []
-    for L, C, r, w in row_kernel_tiles(plan, reverse):
-        tile = dataclasses.replace(plan.tile, L=L, C=C)
+def row_kernel_variants(plan, reverse: bool):
+    """Tiles (as `TileConfig`s) of the candidate builds of the forward kernel (or the reverse scan): every
+    (L, C, R, W) of `row_kernel_tiles`, each with the row sums leaving a step through a store by one lane (a
+    branch per step) and through a store by every lane of the group (no branch: the compiler then overlaps
+    consecutive steps, which costs registers and, on some recurrences, a wave per SIMD); the first tile also
+    with the time loop unrolled four times.  Measured: the forward kernel of Mamba-1 0.195 -> 0.163 ms and of the
+    gated delta rule 3.89 -> 3.51 ms without the branch, that of Mamba-2 0.51 -> 0.61 ms (3 instead of 4 waves
+    per SIMD) unless also unrolled four times (0.49 ms); RWKV-7 the same either way."""
+    bit = 2 if reverse else 1
+    base = plan.tile
+    out = []
+    for k, (L, C, r, w) in enumerate(row_kernel_tiles(plan, reverse)):
+        tile = dataclasses.replace(base, L=L, C=C)
         tile = dataclasses.replace(tile, R1=r, W1=w) if reverse else dataclasses.replace(tile, R=r, W=w)
+        on, off = (base.NB | bit, base.UR), (base.NB & ~bit, base.UR)
+        knobs = [on, off] if base.NB & bit else [off, on]       # (the plan's own setting first)
+        if k == 0 and not (reverse and plan.part.dstep_needs_state):
+            knobs.append((base.NB | bit, 4))
+        for nb, ur in knobs:
+            t = dataclasses.replace(tile, NB=nb, UR=ur)
+            if t not in out:
+                out.append(t)
+    return out
+
+
+def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save: bool = True):
+    """[(spec, path)] for `row_kernel_variants`, compiled side by side (`save=False`: the inference
+    variant of the forward kernel)."""
+    specs, seen_src = [], set()
+    for tile in row_kernel_variants(plan, reverse):
         em = Emitter(dataclasses.replace(plan, tile=tile))
-        specs.append(em.bw1() if reverse else em.fw(save=save))
+        spec = em.bw1() if reverse else em.fw(save=save)
+        if spec.source not in seen_src:
+            seen_src.add(spec.source)
+            specs.append(spec)
     return _compile(specs, force, seen)
 
 

@@ -85,6 +85,12 @@ class TileConfig:
     HB: int = 1          # heads walked by one gradient-kernel instance (sums head-broadcast grads in registers)
     MS: int = 1          # instances sharing the rows of one (batch, head, chunk) in the gradient kernel;
                          # above 1 the row/scalar-input grads are summed across them with atomics
+    WPE: int = 0         # waves per SIMD the row kernels are compiled for (0 = whatever the compiler arrives at)
+    UR: int = 2          # row kernels: unrolling of the loop over the staged timesteps
+    NB: int = 1          # row sums leave a step without a branch (every lane of a group stores them): bit 0 = forward
+                         # kernel, bit 1 = reverse scan.  Lets the compiler overlap consecutive steps, at the price of registers.
+    PF: int = 0          # row kernels: 1 = the operands of a step's first row sum are read from LDS one step ahead, 2 = all
+                         # (measured on RWKV-7: within 2 % of 0 either way; kept as a tuning knob)
 
     @property
     def G(self): return 64 // self.L

@@ -219,6 +219,11 @@ def test_row_kernel_candidate_tiles_are_valid():
                 t = dataclasses.replace(plan.tile, L=L, C=C)
                 t = dataclasses.replace(t, R1=r, W1=w) if reverse else dataclasses.replace(t, R=r, W=w)
                 planner.check_tile(t, plan.H, plan.NP, plan.part)
+            variants = launch.row_kernel_variants(plan, reverse)
+            assert len(variants) >= len(tiles) and len({repr(v) for v in variants}) == len(variants)
+            assert variants[0] == dataclasses.replace(variants[0], NB=plan.tile.NB, UR=plan.tile.UR)     # first: the plan's own tile
+            for v in variants:
+                planner.check_tile(v, plan.H, plan.NP, plan.part)
     assert (8, 16, 2, 8) in launch.row_kernel_tiles(prebuild.plan_for('rwkv7'), False)
 
 

@@ -86,6 +86,17 @@ TILED = [
     # 16 columns per lane (a state row of 128 in 8 lanes: three reduction steps), one workgroup per head
     ('cfg:rwkv7', '1,19,2,128,128', 'bf16', 1, 'L=8,C=16,R=2,W=8,R1=2,W1=8'),
     ('cfg:mamba2', '1,16,2,64,128', 'f32', 0, 'L=8,C=16,R=1,W=8,R1=1,W1=8'),
+    # state rows spread over 32 / 64 lanes: the reductions then use the gfx950 row swaps (emulated by the harness)
+    ('cfg:rwkv7', '1,16,1,8,128', 'f32', 1, 'L=32,C=4,R=1,W=1'),
+    ('cfg:rwkv7', '1,16,1,8,128', 'f32', 0, 'L=64,C=2,R=1,W=1'),
+    # several gradient-kernel instances per wave as consecutive row slices of one chunk (narrow states): ragged slices,
+    # a slice with no row, a partial last chunk; their gradients are summed across the wave before one instance stores
+    ('cfg:mamba1', '2,21,2,37,16', 'f32', 0, 'MS=8'),
+    ('gla', '2,19,2,21,32', 'f32', 1, 'MS=2'),
+    # knobs of the row kernels: branch-free stores of the row sums in both kernels, deeper unrolling, operands read ahead
+    ('cfg:rwkv7', '1,19,1,128,128', 'bf16', 0, 'NB=3,UR=4,PF=1'),
+    ('cfg:mamba2', '1,21,2,64,128', 'f32', 1, 'NB=0,PF=2'),
+    ('cfg:mamba1', '2,16,2,128,16', 'f32', 1, 'NB=3,UR=16'),
 ]
 
 
