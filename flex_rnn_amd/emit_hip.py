@@ -666,6 +666,8 @@ class Emitter:
         body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = 0; tt < nt; tt++) {{\n')
         for nm_ in order:
             body.append(ahead[nm_][1] if nm_ in ahead else self._load_operand(*operands[nm_], R, C, 'tt'))
+        if getattr(t, 'SB', 0):
+            body.append('      __builtin_amdgcn_sched_barrier(0);\n')
         call = []
         for nm_ in used:
             if nm_ in p.in_names:
@@ -834,7 +836,7 @@ class Emitter:
         # `bw_dstep`.  Those without a column extent (one register per row) are loaded once for
         # both, so that the compiler sees common subexpressions of the two calls - typically
         # the exponential of a per-row decay - as such.
-        shared_in = [i for i in used_in if needs_state and self.tdep[i] and not self.in_ext(i)[1]
+        shared_in = [i for i in used_in if needs_state and getattr(t, 'SH', 1) and self.tdep[i] and not self.in_ext(i)[1]
                      and p.in_names[i] in used and p.in_names[i] in re_used]
 
         def operand_loads(tt, names, state_var, ahead=None, order=None):
@@ -877,6 +879,8 @@ class Emitter:
             for nm_ in (order if order is not None else list(loads)):
                 if nm_ in loads:
                     code.append(ahead[nm_][1] if ahead and nm_ in ahead else self._load_operand(*loads[nm_], R, C, tt))
+            if getattr(t, 'SB', 0) and order is not None:
+                code.append('      __builtin_amdgcn_sched_barrier(0);\n')
             return code, call, loads
 
         def dstep_block(tt, state_var, indent='      ', ahead=None, order=None):

@@ -89,6 +89,8 @@ class TileConfig:
     UR: int = 2          # row kernels: unrolling of the loop over the staged timesteps
     NB: int = 1          # row sums leave a step without a branch (every lane of a group stores them): bit 0 = forward
                          # kernel, bit 1 = reverse scan.  Lets the compiler overlap consecutive steps, at the price of registers.
+    SH: int = 1          # reverse scan with state recompute: per-row operands loaded once for recompute and d-step
+    SB: int = 0          # row kernels: 1 = the compiler may not move instructions across the end of a step's LDS reads
     PF: int = 0          # row kernels: 1 = the operands of a step's first row sum are read from LDS one step ahead, 2 = all
                          # (measured on RWKV-7: within 2 % of 0 either way; kept as a tuning knob)
 

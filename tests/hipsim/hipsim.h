@@ -32,6 +32,7 @@ static sim_dim3 threadIdx, blockIdx, blockDim, gridDim;
 #define __shared__ static
 #define __launch_bounds__(...)
 #define __HIP_MEMORY_SCOPE_AGENT 0
+#define __builtin_amdgcn_sched_barrier(mask) ((void)0)      // (a hint to the GPU compiler's scheduler)
 using std::max;
 using std::min;
 
