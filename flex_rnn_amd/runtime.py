@@ -31,19 +31,30 @@ _toolchain = None
 
 
 def toolchain_id() -> str:
-    """What identifies the compiler behind `frnn_compile` (the version lines of `hipcc --version`): a code
-    object built by another compiler release must not be taken from the cache."""
+    """What identifies the compiler behind `frnn_compile`: the ROCm release named in `<rocm>/.info/version` and
+    the resolved path and size of the clang binary hipcc drives.  A code object built by another compiler
+    release must not be taken from the cache.  Read from files, not by running the compiler: a process that
+    already uses the GPU (under a profiler, say) should not start programs it does not have to."""
     global _toolchain
     if _toolchain is None:
         hipcc = os.environ.get('FRNN_HIPCC') or next(
             (p for p in (os.path.join(os.environ.get('ROCM_PATH', '/opt/rocm'), 'bin', 'hipcc'), '/opt/rocm/bin/hipcc')
-             if os.access(p, os.X_OK)), 'hipcc')
+             if os.access(p, os.X_OK)), '')
+        root = os.path.dirname(os.path.dirname(os.path.realpath(hipcc))) if hipcc else ''
+        parts = []
         try:
-            out = subprocess.run([hipcc, '--version'], capture_output=True, text=True, timeout=60).stdout
-            lines = [ln.strip() for ln in out.splitlines() if ln.startswith('HIP version') or 'clang version' in ln]
-            _toolchain = ' | '.join(lines) or 'unknown'
-        except (OSError, subprocess.SubprocessError):
-            _toolchain = 'unknown'
+            with open(os.path.join(root, '.info', 'version')) as f:
+                parts.append('rocm version ' + f.read().strip())
+        except OSError:
+            pass
+        for clang in (os.path.join(root, 'lib', 'llvm', 'bin', 'clang++'), os.path.join(root, 'llvm', 'bin', 'clang++')):
+            try:
+                real = os.path.realpath(clang)
+                parts.append(f'{os.path.basename(real)} {os.path.getsize(real)} bytes')
+                break
+            except OSError:
+                continue
+        _toolchain = ' | '.join(parts) or 'unknown'
     return _toolchain
 
 

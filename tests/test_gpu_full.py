@@ -261,7 +261,7 @@ def test_check_grad_and_benchmark_helpers():
     f = flex_rnn_amd.jit(step)
     err = flex_rnn_amd.check_grad(f, f.naive_fp64, _gpu(xs) + _gpu(ss), verbose=False, tol=1e-4)
     assert err < 1e-4
-    ms = flex_rnn_amd.benchmark(f, _gpu(xs) + _gpu(ss), warmup=2, rep=5, verbose=False)
+    ms = flex_rnn_amd.benchmark(f, _gpu(xs) + _gpu(ss), warmup=5, rep=20, verbose=False)      # (time budgets in ms)
     assert ms > 0
 
 
