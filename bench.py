@@ -217,10 +217,11 @@ def main():
     if name == 'rwkv7' and not args.no_others:
         others = {}
         for other in ('mamba1', 'mamba2', 'gated_delta_rule'):
-            r = measure(other, 10, 3, traffic_records)
+            n_steps, n_warm = (10, 3) if other == 'gated_delta_rule' else (20, 10)     # (short steps: long enough for the clocks to settle)
+            r = measure(other, n_steps, n_warm, traffic_records)
             rf = r['roofline']
             others[other] = {'workload': r['config']['workload'], 'ms_per_step': r['ms_per_step'], 'tokens_per_s': r['value'],
-                             'steps': 10, 'warmup': 3, 'bound': rf['bound'], 'frac': rf['frac'] if rf['bound'] == 'hbm' else rf['step_frac'],
+                             'steps': n_steps, 'warmup': n_warm, 'bound': rf['bound'], 'frac': rf['frac'] if rf['bound'] == 'hbm' else rf['step_frac'],
                              'frac_of': 'algorithmic HBM bytes of the step / 8 TB/s' if rf['bound'] == 'hbm'
                              else 'algorithmic flops of the step / 157.3 TFLOP/s',
                              'dominant_kernel': rf['kernel'], 'dominant_kernel_frac': rf['frac'],

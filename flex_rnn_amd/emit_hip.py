@@ -619,10 +619,18 @@ class Emitter:
         if rfront:
             fn_src = self._stage_row_front(stg, A, rfront, set(used), MT, 'fw_rowpre') + '\n' + fn_src
         body.append(stg.decls() + stg.bases() + stg.zero_pads())
+        # Results of a chunk (outputs, saved row sums) go to LDS per step and from there to memory.  With `df` they leave during
+        # the next chunk, from the other half of a double buffer, and the checkpoint is stored after the staged operands were
+        # written to LDS: a wave that waits for its prefetched loads also waits for every store it has issued, so stores
+        # issued just before that wait put their latency into every chunk.  Measured: forward kernel and reverse scan of the
+        # gated delta rule 3.60 / 3.43 -> 3.34 / 3.13 ms, Mamba-2's forward kernel 0.49 -> 0.46 ms; RWKV-7 0.81 / 0.73 -> 0.86 /
+        # 0.82 ms (its stores then compete with the LDS reads of the steps), so both forms are timed candidates.
+        df = bool(getattr(t, 'DF', 0))
+        nb_ = 2 if df else 1
         for k in range(nout):
-            body.append(f'  __shared__ float s_out{k}[{TS}][{MT}];\n')
+            body.append(f'  __shared__ float s_out{k}[{nb_}][{TS}][{MT}];\n')
         for k in range(naux):
-            body.append(f'  __shared__ float s_aux{k}[{TS}][{MT}];\n')
+            body.append(f'  __shared__ float s_aux{k}[{nb_}][{TS}][{MT}];\n')
         # state
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
@@ -637,17 +645,44 @@ class Emitter:
                 body.append(self._load_const_input(A, i, R, C))
         body.append(stg.load('0', '  '))
         body.append(f'  for (int t0 = 0; t0 < T; t0 += {TS}) {{\n')
-        # checkpoint
-        body.append(f'    if (t0 % {DT} == 0) {{\n')
-        for k in range(nst if save else 0):
-            rr, cc = _dims(st_ext[k], R, C)
-            body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
-                        f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
-                        f'((float*){A.p(f"sck{k}")})[{self._ck_index(f"t0 / {DT}")}] = S{k}[r][c]; }}\n')
-        body.append('    }\n    __syncthreads();\n')
+        def checkpoint():
+            out = [f'    if (t0 % {DT} == 0) {{\n']
+            for k in range(nst if save else 0):
+                rr, cc = _dims(st_ext[k], R, C)
+                out.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                           f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
+                           f'((float*){A.p(f"sck{k}")})[{self._ck_index(f"t0 / {DT}")}] = S{k}[r][c]; }}\n')
+            out.append('    }\n')
+            return out
+
+        def flush(tbase, ntv, buf, ind):
+            """The staged results of the chunk starting at `tbase` (`ntv` timesteps, LDS buffer `buf`) to memory."""
+            out = [f'{ind}for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
+                   f'{ind}  if (m_ < M && tt_ < {ntv}) {{\n']
+            for k in range(nout):
+                dt = DT_CODE[plan.out_dtypes[k]]
+                nm = f'out{k}'
+                out.append(f'{ind}    stf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)({tbase} + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}, s_out{k}[{buf}][tt_][x_]);\n')
+            for k in range(naux):
+                out.append(f'{ind}    ((float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + ({tbase} + tt_)) * M + m_] = s_aux{k}[{buf}][tt_][x_];\n')
+            out.append(f'{ind}  }} }}\n')
+            return out
+
+        if not df:
+            body += checkpoint()
+        body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
         body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
+        if df:
+            body += checkpoint()
+            if nout or naux:        # the chunk before this one (always a whole one)
+                body.append(f'    if (t0 > 0) {{\n')
+                body += flush(f't0 - {TS}', str(TS), f'((t0 / {TS}) & 1) ^ 1', '      ')
+                body.append('    }\n')
+            body.append(f'    const int ob_ = (t0 / {TS}) & 1;\n')
+        else:
+            body.append('    const int ob_ = 0;\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
         # LDS operands of a step, in the order the step needs them; those its first row sum depends on are read one
         # step ahead (the sum, and with it everything else of the step, would otherwise wait for the LDS)
@@ -698,20 +733,20 @@ class Emitter:
         # the next step's LDS reads and state-independent arithmetic with this step
         body.append('      {\n' if getattr(t, 'NB', 1) & 1 else '      if (l == 0) {\n')
         for k in range(nout):
-            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_out{k}[tt][rloc + r] = y{k}[{"r" if rrs > 1 else "0"}][0];\n')
+            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_out{k}[ob_][tt][rloc + r] = y{k}[{"r" if rrs > 1 else "0"}][0];\n')
         for k in range(naux):
-            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_aux{k}[tt][rloc + r] = a{k}[{"r" if rrs > 1 else "0"}][0];\n')
-        body.append('      }\n    }\n    __syncthreads();\n')
-        # flush
-        body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
-                    f'      if (m_ < M && tt_ < nt) {{\n')
-        for k in range(nout):
-            dt = DT_CODE[plan.out_dtypes[k]]
-            nm = f'out{k}'
-            body.append(f'        stf<{dt}>({A.p(nm)}, (i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}, s_out{k}[tt_][x_]);\n')
-        for k in range(naux):
-            body.append(f'        ((float*){A.p("aux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_] = s_aux{k}[tt_][x_];\n')
-        body.append('      } }\n  }\n')
+            body.append(f'#pragma unroll\n        for (int r = 0; r < {R}; r++) s_aux{k}[ob_][tt][rloc + r] = a{k}[{"r" if rrs > 1 else "0"}][0];\n')
+        body.append('      }\n    }\n')
+        if df:
+            body.append('  }\n')
+            if nout or naux:        # the last chunk (possibly a partial one)
+                body.append(f'  if (T > 0) {{ const int tl_ = ((T - 1) / {TS}) * {TS};\n    __syncthreads();\n')
+                body += flush('tl_', 'T - tl_', f'(tl_ / {TS}) & 1', '    ')
+                body.append('  }\n')
+        else:
+            body.append('    __syncthreads();\n')
+            body += flush('t0', 'nt', '0', '    ')
+            body.append('  }\n')
         # final state
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
@@ -779,10 +814,14 @@ class Emitter:
         body.append(stg.decls() + stg.bases() + stg.zero_pads())
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
+        # (as in the forward kernel: with `df` a chunk's column gradients and saved sums leave LDS during the next chunk,
+        # and the d-state checkpoint is stored after the wait for the staged operands)
+        df = bool(getattr(t, 'DF', 0))
+        nb_ = 2 if df else 1
         for i in tdep_col:
-            body.append(f'  __shared__ float s_dc{i}[{TS}][{MT}];\n')
+            body.append(f'  __shared__ float s_dc{i}[{nb_}][{TS}][{MT}];\n')
         for k in range(ndaux):
-            body.append(f'  __shared__ float s_da{k}[{TS}][{MT}];\n')
+            body.append(f'  __shared__ float s_da{k}[{nb_}][{TS}][{MT}];\n')
         # incoming cotangent of the final state
         for k in range(nst):
             rr, cc = _dims(st_ext[k], R, C)
@@ -815,14 +854,39 @@ class Emitter:
             body.append(f'  float pS{k}[{rr}][{cc}];\n' + ckpt_fetch(k, f'tlast / {DT}', '  '))
         body.append(f'  for (int t0 = tlast; t0 >= 0; t0 -= {TS}) {{\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
-        # d_state checkpoints are only read by the gradient kernel
-        body.append(f'    if ((t0 + {TS}) % {DT} == 0{f" || t0 + {TS} >= T" if self.tail_dt else ""}) {{\n')
-        for k in range(nst if needs_gradient_kernel(p) else 0):
-            rr, cc = _dims(st_ext[k], R, C)
-            body.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
-                        f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
-                        f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"t0 / {DT}")}] = D{k}[r][c]; }}\n')
-        body.append('    }\n    __syncthreads();\n')
+        def d_checkpoint():
+            # d_state checkpoints are only read by the gradient kernel
+            out = [f'    if ((t0 + {TS}) % {DT} == 0{f" || t0 + {TS} >= T" if self.tail_dt else ""}) {{\n']
+            for k in range(nst if needs_gradient_kernel(p) else 0):
+                rr, cc = _dims(st_ext[k], R, C)
+                out.append(f'#pragma unroll\n      for (int r = 0; r < {rr}; r++) if (row0 + r < M) {{\n'
+                           f'#pragma unroll\n        for (int c = 0; c < {cc}; c++) '
+                           f'((float*){A.p(f"dck{k}")})[{self._ck_index(f"t0 / {DT}")}] = D{k}[r][c]; }}\n')
+            out.append('    }\n')
+            return out
+
+        def flush(tbase, ntv, buf, ind):
+            """Column gradients and saved sums of the chunk starting at `tbase` (`ntv` timesteps, LDS buffer `buf`) to memory."""
+            if not (tdep_col or ndaux):
+                return []
+            out = [f'{ind}for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
+                   f'{ind}  if (m_ < M && tt_ < {ntv}) {{\n']
+            for i in tdep_col:
+                nm = f'din{i}'
+                idx = f'(i64)b * {A.s(nm, 0)} + (i64)({tbase} + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}'
+                if i in self.atomic:
+                    out.append(f'{ind}    atomic_addf({A.p(nm)}, {idx}, s_dc{i}[{buf}][tt_][x_]);\n')
+                else:
+                    dt = DT_CODE[plan.in_dtypes[i]]
+                    out.append(f'{ind}    stf<{dt}>({A.p(nm)}, {idx}, s_dc{i}[{buf}][tt_][x_]);\n')
+            for k in range(ndaux):
+                out.append(f'{ind}    ((float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + ({tbase} + tt_)) * M + m_] = s_da{k}[{buf}][tt_][x_];\n')
+            out.append(f'{ind}  }} }}\n')
+            return out
+
+        if not df:
+            body += d_checkpoint()
+        body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
         for k in range(nst if needs_state else 0):
@@ -831,6 +895,16 @@ class Emitter:
                         f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = pS{k}[r][c];\n')
         body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ')
                     + ''.join(ckpt_fetch(k, f't0 / {DT} - 1', '      ') for k in range(nst if needs_state else 0)) + '    }\n')
+        if df:
+            body += d_checkpoint()
+            pre = flush(f't0 + {TS}', f'min({TS}, T - (t0 + {TS}))' if tail else str(TS), f'((t0 / {TS}) & 1) ^ 1', '      ')
+            if pre:                 # the chunk walked before this one (the later timesteps; only that one can be partial)
+                body.append('    if (t0 < tlast) {\n')
+                body += pre
+                body.append('    }\n')
+            body.append(f'    const int ob_ = (t0 / {TS}) & 1;\n')
+        else:
+            body.append('    const int ob_ = 0;\n')
 
         # With state recompute a timestep's operands are read by `bw_restep` and again by
         # `bw_dstep`.  Those without a column extent (one register per row) are loaded once for
@@ -910,9 +984,9 @@ class Emitter:
             code.append(f'{indent}{{\n' if getattr(t, 'NB', 1) & 2 else f'{indent}if (l == 0) {{\n')
             ridx = 'r' if rrs > 1 else '0'
             for i in tdep_col:
-                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_dc{i}[{tt}][rloc + r] = gc{i}[{ridx}][0];\n')
+                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_dc{i}[ob_][{tt}][rloc + r] = gc{i}[{ridx}][0];\n')
             for k in range(ndaux):
-                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_da{k}[{tt}][rloc + r] = da{k}[{ridx}][0];\n')
+                code.append(f'#pragma unroll\n{indent}  for (int r = 0; r < {R}; r++) s_da{k}[ob_][{tt}][rloc + r] = da{k}[{ridx}][0];\n')
             code.append(f'{indent}}}\n')
             return code
 
@@ -948,23 +1022,17 @@ class Emitter:
                 body.append(f'    if ({tt} < nt) {{\n' if tail else '    {\n')
                 body += dstep_block(str(tt), lambda k, tt=tt: f'Sh{k}_{tt}')
                 body.append('    }\n')
-        body.append('    __syncthreads();\n')
-        # flush column grads and daux
-        if tdep_col or ndaux:
-            body.append(f'    for (int e_ = tid; e_ < {TS * MT}; e_ += {NT}) {{ int tt_ = e_ / {MT}, x_ = e_ % {MT}; int m_ = mt * {MT} + x_;\n'
-                        f'      if (m_ < M && tt_ < nt) {{\n')
-            for i in tdep_col:
-                nm = f'din{i}'
-                idx = f'(i64)b * {A.s(nm, 0)} + (i64)(t0 + tt_) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + (i64)m_ * {A.s(nm, 3)}'
-                if i in self.atomic:
-                    body.append(f'        atomic_addf({A.p(nm)}, {idx}, s_dc{i}[tt_][x_]);\n')
-                else:
-                    dt = DT_CODE[plan.in_dtypes[i]]
-                    body.append(f'        stf<{dt}>({A.p(nm)}, {idx}, s_dc{i}[tt_][x_]);\n')
-            for k in range(ndaux):
-                body.append(f'        ((float*){A.p("daux")})[((((i64){k} * A.B + b) * H + h) * T + (t0 + tt_)) * M + m_] = s_da{k}[tt_][x_];\n')
-            body.append('      } }\n')
-        body.append('  }\n')
+        if df:
+            body.append('  }\n')
+            last = flush('0', f'min({TS}, T)' if tail else str(TS), '0', '    ')
+            if last:                # the chunk walked last: timesteps 0 .. TS-1
+                body.append('  if (T > 0) {\n    __syncthreads();\n')
+                body += last
+                body.append('  }\n')
+        else:
+            body.append('    __syncthreads();\n')
+            body += flush('t0', 'nt', '0', '    ')
+            body.append('  }\n')
         for i in const_col:
             nm = f'din{i}'
             body.append(f'  if (l == 0) {{\n#pragma unroll\n    for (int r = 0; r < {R}; r++) if (row0 + r < M) '

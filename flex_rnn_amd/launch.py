@@ -159,34 +159,42 @@ def row_kernel_tiles(plan, reverse: bool):
     return out
 
 
+TUNE_KNOBS_FROM = 1 << 26       # state-element timesteps from which the row kernels' code-generation knobs are timed too
+
+
 def row_kernel_variants(plan, reverse: bool):
     """Tiles (as `TileConfig`s) of the candidate builds of the forward kernel (or the reverse scan): every
-    (L, C, R, W) of `row_kernel_tiles`, each with the row sums leaving a step through a store by one lane (a
-    branch per step) and through a store by every lane of the group (no branch: the compiler then overlaps
-    consecutive steps, which costs registers and, on some recurrences, a wave per SIMD); the first tile also
-    with the time loop unrolled four times.  Measured: the forward kernel of Mamba-1 0.195 -> 0.163 ms and of the
-    gated delta rule 3.89 -> 3.51 ms without the branch, that of Mamba-2 0.51 -> 0.61 ms (3 instead of 4 waves
-    per SIMD) unless also unrolled four times (0.49 ms); RWKV-7 the same either way."""
+    (L, C, R, W) of `row_kernel_tiles`; for problems of `TUNE_KNOBS_FROM` state-element timesteps or more each of
+    them in four forms - the row sums leaving a step through a store by one lane (a branch per step) or by
+    every lane of the group (no branch: the compiler then overlaps consecutive steps, which costs registers
+    and, on some recurrences, a wave per SIMD), and a chunk's results leaving LDS at once or during the next
+    chunk (`TileConfig.DF`) - and the first tile also with the time loop unrolled four times.  Measured: the
+    forward kernel of Mamba-1 0.195 -> 0.163 ms and of the gated delta rule 3.89 -> 3.51 ms without the branch,
+    that of Mamba-2 0.51 -> 0.61 ms (3 instead of 4 waves per SIMD) unless also unrolled four times (0.49 ms);
+    RWKV-7 the same either way."""
     bit = 2 if reverse else 1
     base = plan.tile
+    big = plan.B * plan.T * plan.H * plan.M * plan.NP >= TUNE_KNOBS_FROM
     out = []
     for k, (L, C, r, w) in enumerate(row_kernel_tiles(plan, reverse)):
         tile = dataclasses.replace(base, L=L, C=C)
         tile = dataclasses.replace(tile, R1=r, W1=w) if reverse else dataclasses.replace(tile, R=r, W=w)
-        on, off = (base.NB | bit, base.UR), (base.NB & ~bit, base.UR)
-        knobs = [on, off] if base.NB & bit else [off, on]       # (the plan's own setting first)
-        if k == 0 and not (reverse and plan.part.dstep_needs_state):
-            knobs.append((base.NB | bit, 4))
-        for nb, ur in knobs:
-            t = dataclasses.replace(tile, NB=nb, UR=ur)
+        own = (base.NB, base.DF, base.UR)               # (the plan's own setting first)
+        knobs = [own]
+        if big:
+            knobs += [(base.NB ^ bit, base.DF, base.UR), (base.NB, base.DF ^ 1, base.UR), (base.NB ^ bit, base.DF ^ 1, base.UR)]
+            if k == 0 and not (reverse and plan.part.dstep_needs_state):
+                knobs.append((base.NB | bit, base.DF, 4))
+        for nb, df, ur in knobs:
+            t = dataclasses.replace(tile, NB=nb, DF=df, UR=ur)
             if t not in out:
                 out.append(t)
     return out
 
 
-def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save: bool = True):
-    """[(spec, path)] for `row_kernel_variants`, compiled side by side (`save=False`: the inference
-    variant of the forward kernel)."""
+def row_kernel_specs(plan, reverse: bool, save: bool = True):
+    """Kernel sources of `row_kernel_variants` (`save=False`: the inference variant of the forward kernel),
+    without duplicates; nothing is compiled."""
     specs, seen_src = [], set()
     for tile in row_kernel_variants(plan, reverse):
         em = Emitter(dataclasses.replace(plan, tile=tile))
@@ -194,7 +202,12 @@ def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save:
         if spec.source not in seen_src:
             seen_src.add(spec.source)
             specs.append(spec)
-    return _compile(specs, force, seen)
+    return specs
+
+
+def row_kernel_builds(plan, reverse: bool, force: bool = False, seen=None, save: bool = True):
+    """[(spec, path)] for `row_kernel_specs`, compiled side by side."""
+    return _compile(row_kernel_specs(plan, reverse, save), force, seen)
 
 
 def compile_plan(plan, force: bool = False, seen=None) -> List[Tuple[KernelSpec, str]]:
@@ -325,25 +338,57 @@ class CompiledPlan:
         self.builds, self.build_times, self._grid, self._packer = {}, {}, {}, {}
         if plan.B == 0 or plan.T == 0:
             return                          # nothing will ever be launched for an empty batch or no timesteps
-        # Every kernel comes in a few candidate builds (tiles of the row kernels; prefetch depth and
-        # occupancy request of the gradient kernel), first-ranked first.  All are loaded; the first
-        # call that runs a kernel times its candidates on that call's tensors and keeps the fastest.
+        # Every kernel comes in a few candidate builds (tiles and code-generation knobs of the row kernels; prefetch
+        # depth and occupancy request of the gradient kernel), first-ranked first.  The first call that runs a kernel
+        # times its candidates on that call's tensors and keeps the fastest; the choice is stored (`PICKS`).  Where a
+        # stored choice exists for a row kernel, only that candidate is compiled and loaded.
+        self._tune_on = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
+        self._fixed = _fixed_picks()
+        self._device_name()                                     # (asked for here, not on the compiler threads below)
         with ThreadPoolExecutor(max_workers=3) as pool:         # compiler runs; loading happens on this thread
-            jobs = {'frnn_fw': pool.submit(lambda: [(s_, p_, None) for s_, p_ in row_kernel_builds(plan, False)]),
-                    'frnn_bw1': pool.submit(lambda: [(s_, p_, None) for s_, p_ in row_kernel_builds(plan, True)])}
+            jobs = {'frnn_fw': pool.submit(self._row_builds, 'frnn_fw', row_kernel_specs(plan, False)),
+                    'frnn_bw1': pool.submit(self._row_builds, 'frnn_bw1', row_kernel_specs(plan, True))}
             if needs_gradient_kernel(plan.part):
-                jobs['frnn_bw2'] = pool.submit(gradient_kernel_builds, plan)
+                jobs['frnn_bw2'] = pool.submit(lambda: (gradient_kernel_builds(plan), None))
             built = {k: j.result() for k, j in jobs.items()}
+        for k, (v, chosen) in built.items():
+            self._install(k, v, chosen)
+
+    def _device_name(self):
+        """Name of the GPU the plan is loaded on (part of the key under which timed choices are stored)."""
+        if getattr(self, '_dev_name', None) is None:
+            on_gpu = self.device is not None and self.device.type == 'cuda'
+            if on_gpu:
+                idx = self.device.index if self.device.index is not None else th.cuda.current_device()
+                self._dev_name = th.cuda.get_device_name(idx)
+            else:
+                self._dev_name = str(self.device)
+        return self._dev_name
+
+    def _row_builds(self, name, specs):
+        """([(spec, path or None, None)], stored choice or None) for the candidate sources of a row kernel: with a
+        stored choice (and no request to time again) only the chosen candidate is compiled."""
+        rec = None
+        if self._tune_on and name not in self._fixed and len(specs) > 1 and os.environ.get('FLEX_RNN_RETUNE', '0') == '0':
+            rec = PICKS.get(PICKS.key(name, [(s_, None, None) for s_ in specs], self._device_name(), self.plan), len(specs))
+        if rec is not None:
+            (spec, path), = _compile([specs[rec['index']]], False, None)
+            return [(s_, path if i == rec['index'] else None, None) for i, s_ in enumerate(specs)], rec
+        return [(s_, p_, None) for s_, p_ in _compile(specs, False, None)], None
+
+    def _install(self, name, built, chosen=None):
+        """Loads the built candidates of kernel `name` (those without a code object stay unloaded) and selects
+        the stored choice, the one named by FLEX_RNN_PICK, or the first; marks the kernel for timing otherwise."""
         on_gpu = self.device is not None and self.device.type == 'cuda'
         with (th.cuda.device(self.device) if on_gpu else contextlib.nullcontext()):
-            self.builds = {k: [(s_, load(s_, p_), r_) for s_, p_, r_ in v] for k, v in built.items()}
-        self.build_times = {}
-        tune = os.environ.get('FLEX_RNN_TUNE', '1') != '0'
-        picks = _fixed_picks()
-        self._tune_pending = {k for k, v in self.builds.items() if tune and len(v) > 1 and k not in picks}
-        self._grid, self._packer = {}, {}
-        for k, v in self.builds.items():
-            self._select(k, picks.get(k, 0))
+            self.builds[name] = [(s_, self._load(s_, p_) if p_ is not None else None, r_) for s_, p_, r_ in built]
+        if chosen is not None:
+            self.build_times[name] = [float('inf') if t is None else t for t in chosen.get('ms', [])] or None
+            self._select(name, chosen['index'])
+            return
+        if len(built) > 1 and self._tune_on and name not in self._fixed:
+            self._tune_pending = set(self._tune_pending) | {name}
+        self._select(name, self._fixed.get(name, 0))
 
     @property
     def bw2_builds(self):
@@ -370,15 +415,6 @@ class CompiledPlan:
         env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
         self._grid[name] = tuple(int(eval(g, {}, env)) for g in spec.grid)
         self._packer[name] = struct.Struct('<' + 'q5q' * max(len(spec.tensors), 1) + '5q')
-
-    def _add_builds(self, name, built):
-        on_gpu = self.device is not None and self.device.type == 'cuda'
-        with (th.cuda.device(self.device) if on_gpu else contextlib.nullcontext()):
-            self.builds[name] = [(s_, self._load(s_, p_), r_) for s_, p_, r_ in built]
-        picks = _fixed_picks()
-        if len(built) > 1 and os.environ.get('FLEX_RNN_TUNE', '1') != '0' and name not in picks:
-            self._tune_pending.add(name)
-        self._select(name, picks.get(name, 0))
 
     # ------------------------------------------------------------------ launch helper
     def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
@@ -467,8 +503,7 @@ class CompiledPlan:
             return
         self._tune_pending.discard(name)
         n = len(self.builds[name])
-        dev = next(t.device for t in tensors.values() if t.is_cuda)
-        pkey = PICKS.key(name, self.builds[name], th.cuda.get_device_name(dev), self.plan)
+        pkey = PICKS.key(name, self.builds[name], self._device_name(), self.plan)
         rec = PICKS.get(pkey, n) if os.environ.get('FLEX_RNN_RETUNE', '0') == '0' else None
         if rec is not None:                     # chosen before (by this or an earlier process): no timing
             self._select(name, rec['index'])
@@ -533,7 +568,7 @@ class CompiledPlan:
         """Outputs and final states only (inference): a forward kernel that writes no checkpoints and
         no saved row sums, built on first use."""
         if 'frnn_fwi' not in self.kernels and self.plan.B and self.plan.T:
-            self._add_builds('frnn_fwi', [(s_, p_, None) for s_, p_ in row_kernel_builds(self.plan, False, save=False)])
+            self._install('frnn_fwi', *self._row_builds('frnn_fwi', row_kernel_specs(self.plan, False, save=False)))
         pl, p = self.plan, self.plan.part
         dev = inputs[0].device
         outs = tuple(th.empty(pl.B, pl.T, pl.H, pl.M, dtype=dt, device=dev) for dt in pl.out_dtypes)

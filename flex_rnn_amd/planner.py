@@ -89,6 +89,9 @@ class TileConfig:
     UR: int = 2          # row kernels: unrolling of the loop over the staged timesteps
     NB: int = 1          # row sums leave a step without a branch (every lane of a group stores them): bit 0 = forward
                          # kernel, bit 1 = reverse scan.  Lets the compiler overlap consecutive steps, at the price of registers.
+    DF: int = 0          # row kernels: 1 = a chunk's results leave LDS during the next chunk (double buffer) and checkpoints are
+                         # stored after the wait for the staged operands, so that a wave's stores have a chunk's time to complete
+                         # before it next waits for its prefetched loads.  Pays on some recurrences only; a timed candidate.
     SH: int = 1          # reverse scan with state recompute: per-row operands loaded once for recompute and d-step
     SB: int = 0          # row kernels: 1 = the compiler may not move instructions across the end of a step's LDS reads
     PF: int = 0          # row kernels: 1 = the operands of a step's first row sum are read from LDS one step ahead, 2 = all

@@ -67,10 +67,6 @@ class SimPlan(CompiledPlan):
         for spec in specs:
             self._add_kernel(spec)
 
-    def _add_builds(self, name, built):
-        if name not in self.kernels:
-            self._add_kernel(built[0][0])
-
     def _tune(self, name, tensors, accumulators=()):
         pass
 

@@ -252,3 +252,11 @@ def test_timed_picks_are_kept_beside_the_cache(tmp_path, monkeypatch):
     assert b.get(key, 2) is None              # a stored index that the candidate list no longer has is ignored
     b.put('other', 0, [1.0])
     assert launch._Picks().get(key, 3)['index'] == 2 and launch._Picks().get('other', 1)['index'] == 0
+
+
+def test_compiled_plan_keeps_its_host_interface():
+    """The host object behind `forward` / `backward` (the CPU harness swaps only its two device-facing methods)."""
+    from flex_rnn_amd.launch import CompiledPlan
+    for m in ('_launch', '_tune', '_select', '_register', '_install', '_row_builds', 'forward', 'forward_only', 'backward',
+              'static_layout', 'launch_static'):
+        assert callable(getattr(CompiledPlan, m, None)), m
