@@ -518,9 +518,9 @@ class Emitter:
 
     @staticmethod
     def _operand_order(g: Graph, names, skip=()):
-        """(early, order): `early` = those of the graph inputs `names` that the first row sum of `g` depends on
-        (a step cannot start before it has them), `order` = all of `names`, the early ones first, the rest by
-        first use.  States (`skip`) are registers, not LDS operands."""
+        """The graph inputs `names` in the order a step of `g` needs them: first those that its first row sum
+        depends on (a step cannot start before it has them), then the rest by first use.  States (`skip`) are
+        registers, not LDS operands."""
         nm = g.node_map()
         first = next((n for n in g.nodes if n.op == 'sum'), None)
         seen = set()
@@ -538,30 +538,19 @@ class Emitter:
             for a in n.value_args():
                 pos.setdefault(a, k)
         rest = sorted((v for v in names if v not in early), key=lambda v: pos.get(v, len(g.nodes)))
-        return early, early + rest
+        return early + rest
 
-    def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str, decl: bool = True) -> str:
+    def _load_operand(self, var: str, sname: str, ext, R: int, C: int, tt: str) -> str:
         """Registers <- staged LDS operand for timestep tt."""
-        rr, cc = _dims(ext, R, C)
         if ext == (False, True):
-            return ((f'      float {var}[1][{C}];\n' if decl else '') + f'#pragma unroll\n      for (int c = 0; c < {C}; c++) '
+            return (f'      float {var}[1][{C}];\n#pragma unroll\n      for (int c = 0; c < {C}; c++) '
                     f'{var}[0][c] = {sname}[{tt}][COL(c)];\n')
         if ext == (True, False):
-            return ((f'      float {var}[{R}][1];\n' if decl else '') + f'#pragma unroll\n      for (int r = 0; r < {R}; r++) '
+            return (f'      float {var}[{R}][1];\n#pragma unroll\n      for (int r = 0; r < {R}; r++) '
                     f'{var}[r][0] = {sname}[{tt}][rloc + r];\n')
         if ext == (False, False):
-            return (f'      float {var}[1][1]; ' if decl else '      ') + f'{var}[0][0] = {sname}[{tt}][0];\n'
+            return f'      float {var}[1][1]; {var}[0][0] = {sname}[{tt}][0];\n'
         raise AssertionError
-
-    def _ahead_operand(self, var: str, sname: str, ext, R: int, C: int, nxt: str):
-        """An operand that is read from LDS one step ahead.  Returns (code before the time loop: the first
-        step's value into `<var>n`; code inside the loop: this step's value out of `<var>n` into `var`, and the
-        next step's - staged timestep `nxt`, clamped to the staged range by the caller - into `<var>n`)."""
-        rr, cc = _dims(ext, R, C)
-        copy = (f'      float {var}[{rr}][{cc}];\n#pragma unroll\n      for (int r = 0; r < {rr}; r++)\n#pragma unroll\n'
-                f'      for (int c = 0; c < {cc}; c++) {var}[r][c] = {var}n[r][c];\n')
-        return (lambda first: self._load_operand(f'{var}n', sname, ext, R, C, first),
-                copy + self._load_operand(f'{var}n', sname, ext, R, C, nxt, decl=False))
 
     def _load_const_input(self, A: _Args, i: int, R: int, C: int) -> str:
         """Time-independent input -> registers, once."""
@@ -684,8 +673,7 @@ class Emitter:
         else:
             body.append('    const int ob_ = 0;\n')
         body.append(f'    const int nt = {f"min({TS}, T - t0)" if tail else TS};\n')
-        # LDS operands of a step, in the order the step needs them; those its first row sum depends on are read one
-        # step ahead (the sum, and with it everything else of the step, would otherwise wait for the LDS)
+        # LDS operands of a step, in the order the step needs them (those its first row sum depends on first)
         operands = {}                       # graph input -> (register array, LDS array, extent)
         for nm_ in used:
             if nm_ in p.in_names and self.tdep[p.in_names.index(nm_)]:
@@ -693,16 +681,10 @@ class Emitter:
                 operands[nm_] = (f'x{i}', f's_in{i}', self.in_ext(i))
             elif nm_ in rfront:
                 operands[nm_] = (f'd{rfront.index(nm_)}', f's_d{rfront.index(nm_)}', (False, True))
-        early, order = self._operand_order(g, list(operands), skip=p.st_names)
-        early = {0: [], 1: early}.get(getattr(t, 'PF', 1), order)          # (PF = 2: every operand a step ahead)
-        ahead = {nm_: self._ahead_operand(*operands[nm_], R, C, f'min(tt + 1, {TS - 1})') for nm_ in early}
-        for nm_ in early:
-            body.append(ahead[nm_][0]('0'))
+        order = self._operand_order(g, list(operands), skip=p.st_names)
         body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = 0; tt < nt; tt++) {{\n')
         for nm_ in order:
-            body.append(ahead[nm_][1] if nm_ in ahead else self._load_operand(*operands[nm_], R, C, 'tt'))
-        if getattr(t, 'SB', 0):
-            body.append('      __builtin_amdgcn_sched_barrier(0);\n')
+            body.append(self._load_operand(*operands[nm_], R, C, 'tt'))
         call = []
         for nm_ in used:
             if nm_ in p.in_names:
@@ -913,9 +895,9 @@ class Emitter:
         shared_in = [i for i in used_in if needs_state and getattr(t, 'SH', 1) and self.tdep[i] and not self.in_ext(i)[1]
                      and p.in_names[i] in used and p.in_names[i] in re_used]
 
-        def operand_loads(tt, names, state_var, ahead=None, order=None):
+        def operand_loads(tt, names, state_var, order=None):
             """Loads of the LDS operands among `names` for timestep `tt` and the argument list.  With `order` the
-            loads come in that order; those in `ahead` were read one step earlier (see `_ahead_operand`)."""
+            loads come in that order."""
             code, call, loads = [], [], {}
             for nm_ in names:
                 if nm_ in p.in_names:
@@ -952,13 +934,11 @@ class Emitter:
                     raise AssertionError(nm_)
             for nm_ in (order if order is not None else list(loads)):
                 if nm_ in loads:
-                    code.append(ahead[nm_][1] if ahead and nm_ in ahead else self._load_operand(*loads[nm_], R, C, tt))
-            if getattr(t, 'SB', 0) and order is not None:
-                code.append('      __builtin_amdgcn_sched_barrier(0);\n')
+                    code.append(self._load_operand(*loads[nm_], R, C, tt))
             return code, call, loads
 
-        def dstep_block(tt, state_var, indent='      ', ahead=None, order=None):
-            code, call, _ = operand_loads(tt, used, state_var, ahead, order)
+        def dstep_block(tt, state_var, indent='      ', order=None):
+            code, call, _ = operand_loads(tt, used, state_var, order)
             for k in range(nst):
                 rr, cc = _dims(st_ext[k], R, C)
                 code.append(f'{indent}float nD{k}[{rr}][{cc}];\n')
@@ -991,16 +971,12 @@ class Emitter:
             return code
 
         if not needs_state:
-            # operands in the order the step needs them; those of its first row sum are read one step ahead
+            # operands in the order the step needs them
             no_state = lambda k: (_ for _ in ()).throw(AssertionError())
             _, _, loads = operand_loads('tt', used, no_state)
-            early, order = self._operand_order(g, list(loads), skip=p.dnst_names)
-            early = {0: [], 1: early}.get(getattr(t, 'PF', 1), order)      # (PF = 2: every operand a step ahead)
-            ahead = {nm_: self._ahead_operand(*loads[nm_], R, C, 'max(tt - 1, 0)') for nm_ in early}
-            for nm_ in early:
-                body.append(ahead[nm_][0]('nt - 1'))
+            order = self._operand_order(g, list(loads), skip=p.dnst_names)
             body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = nt - 1; tt >= 0; tt--) {{\n')
-            body += dstep_block('tt', no_state, ahead=ahead, order=order)
+            body += dstep_block('tt', no_state, order=order)
             body.append('    }\n')
         else:
             # recompute the DT states of this chunk from its checkpoint, then walk back

@@ -93,8 +93,6 @@ class TileConfig:
                          # stored after the wait for the staged operands, so that a wave's stores have a chunk's time to complete
                          # before it next waits for its prefetched loads.  Pays on some recurrences only; a timed candidate.
     SH: int = 1          # reverse scan with state recompute: per-row operands loaded once for recompute and d-step
-    SB: int = 0          # row kernels: 1 = the compiler may not move instructions across the end of a step's LDS reads
-    PF: int = 0          # row kernels: 1 = the operands of a step's first row sum are read from LDS one step ahead, 2 = all
                          # (measured on RWKV-7: within 2 % of 0 either way; kept as a tuning knob)
 
     @property

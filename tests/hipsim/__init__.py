@@ -37,7 +37,9 @@ extern "C" int sim_launch_{spec.name}(const void* argbuf, int gx, int gy, int gz
 extern "C" int sim_args_size_{spec.name}() {{ return (int)sizeof(Args); }}
 '''
     hdr = open(os.path.join(_HERE, 'hipsim.h')).read()
-    key = hashlib.sha256((hdr + src).encode()).hexdigest()[:20]
+    # HIPSIM_BOUNDS=1: every index into a declared array (registers, LDS) is checked, a bad one traps
+    extra = ['-fsanitize=bounds', '-fsanitize-undefined-trap-on-error'] if os.environ.get('HIPSIM_BOUNDS', '0') == '1' else []
+    key = hashlib.sha256((hdr + src + ' '.join(extra)).encode()).hexdigest()[:20]
     os.makedirs(_CACHE, exist_ok=True)
     so = os.path.join(_CACHE, f'{spec.name}_{key}.so')
     if not os.path.isfile(so):
@@ -45,7 +47,7 @@ extern "C" int sim_args_size_{spec.name}() {{ return (int)sizeof(Args); }}
         with open(cpp, 'w') as f:
             f.write(src)
         tmp = so + f'.tmp{os.getpid()}'
-        cmd = ['g++', '-O1', '-std=c++17', '-shared', '-fPIC', '-w', '-I', _HERE, cpp, '-o', tmp]
+        cmd = ['g++', '-O1', '-std=c++17', '-shared', '-fPIC', '-w', *extra, '-I', _HERE, cpp, '-o', tmp]
         subprocess.run(cmd, check=True)
         os.replace(tmp, so)
     return so

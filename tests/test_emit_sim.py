@@ -93,10 +93,21 @@ TILED = [
     # a slice with no row, a partial last chunk; their gradients are summed across the wave before one instance stores
     ('cfg:mamba1', '2,21,2,37,16', 'f32', 0, 'MS=8'),
     ('gla', '2,19,2,21,32', 'f32', 1, 'MS=2'),
-    # knobs of the row kernels: branch-free stores of the row sums in both kernels, deeper unrolling, operands read ahead
-    ('cfg:rwkv7', '1,19,1,128,128', 'bf16', 0, 'NB=3,UR=4,PF=1'),
-    ('cfg:mamba2', '1,21,2,64,128', 'f32', 1, 'NB=0,PF=2'),
+    # knobs of the row kernels: branch-free stores of the row sums in both kernels, deeper unrolling
+    ('cfg:rwkv7', '1,19,1,128,128', 'bf16', 0, 'NB=3,UR=4'),
+    ('cfg:mamba2', '1,21,2,64,128', 'f32', 1, 'NB=0'),
     ('cfg:mamba1', '2,16,2,128,16', 'f32', 1, 'NB=3,UR=16'),
+    # results leave LDS one chunk later (double-buffered staging, checkpoints stored after the staging wait): partial last
+    # chunk, a single chunk, a single timestep, reverse scan with state recompute, vector state, padded width
+    ('cfg:rwkv7', '1,37,1,128,128', 'f32', 0, 'DF=1'),
+    ('cfg:rwkv7', '1,37,2,16,16', 'bf16', 1, 'DF=1,TS=4,DT=4'),
+    ('cfg:mamba1', '2,13,2,128,16', 'f32', 1, 'DF=1'),
+    ('cfg:mamba2', '1,21,2,64,128', 'bf16', 0, 'DF=1,NB=3'),
+    ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1, 'DF=1'),
+    ('cfg:gated_delta_rule', '1,9,1,16,80', 'f32', 0, 'DF=1'),
+    ('cfg:gated_delta_rule', '1,100,2,128,128', 'bf16', 1, 'DF=1,NB=0'),
+    ('rwkv4', '2,11,1,32,1', 'f32', 0, 'DF=1'),
+    ('s4d', '2,8,1,8,6', 'f32', 1, 'DF=1'),
 ]
 
 

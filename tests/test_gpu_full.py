@@ -8,10 +8,11 @@ import pytest
 import torch as th
 
 import flex_rnn_amd
-from flex_rnn_amd import configs, ops
+from flex_rnn_amd import configs, ops, prebuild
 from oracle import recurrence
 
 import cases
+import warm
 
 pytestmark = pytest.mark.gpu
 TOL = {th.float32: 1e-4, th.bfloat16: 1e-2}
@@ -213,6 +214,26 @@ def test_single_timestep_with_a_matrix_input_in_bf16(name):
     want = recurrence.loop_with_grads(step, xs, ss, dys[:1], dys[1:], dtype=th.float64)
     ref = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
     recurrence.assert_all_close(list(out) + list(grads), ref, 1e-2, name)
+
+
+_OFF = pytest.mark.skip(reason='ended in a GPU memory fault (reported while the gradient-kernel candidates were timed) '
+                               'whose cause was not found: the same kernels pass on the CPU harness with guard pages and '
+                               'array bounds checks.  The two experimental knobs of this case (operand read-ahead, scheduling '
+                               'barrier) were taken out of the emitter afterwards; the case stays off the GPU')
+
+
+@pytest.mark.parametrize('name,dims,knobs', warm.KNOB_CASES + [
+    pytest.param('mamba2', (2, 19, 4, 64, 128), 'DF=1,PF=1,SB=1', marks=_OFF)])
+def test_row_kernel_knobs_against_oracle(name, dims, knobs, monkeypatch):
+    """The code-generation knobs of the row kernels that are timed candidates at the benchmark sizes (branch-free
+    row sums, deferred output flush, deeper unrolling), forced at small sizes with a partial last chunk: outputs,
+    final state and all gradients against the oracle."""
+    print(f'case knobs {name} {dims} {knobs}', flush=True)
+    monkeypatch.setenv('FLEX_RNN_TILE', knobs)
+    from test_gpu_parity import run_case
+    errs, got, wl = run_case(name, dims, None)
+    tile = prebuild.plan_for(name, dims).tile
+    assert all(getattr(tile, k) == int(v) for k, v in (kv.split('=') for kv in knobs.split(',')))
 
 
 @pytest.mark.parametrize('name', ['rwkv7', 'mamba1', 'mamba2'])

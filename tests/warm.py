@@ -47,6 +47,10 @@ def no_alloc_tile(name, dims):
     return dataclasses.replace(prebuild.plan_for(name, dims).tile, MS=1)
 
 
+# row-kernel code-generation knobs that the size of the test shapes would not make candidates (tests/test_gpu_full.py)
+KNOB_CASES = [('rwkv7', (2, 37, 2, 64, 64), 'DF=1,NB=3,UR=4'), ('mamba1', (2, 45, 4, 128, 16), 'DF=1,NB=3')]
+
+
 EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
 
 
@@ -82,6 +86,13 @@ def warm(force=False, seen=None):
     from flex_rnn_amd import runtime
     runtime.compile_kernel('probe', NO_ALLOC_PROBE, force=force)
     plans = example_plans()
+    for name, dims, knobs in KNOB_CASES:
+        old = os.environ.get('FLEX_RNN_TILE')
+        os.environ['FLEX_RNN_TILE'] = knobs
+        try:
+            plans.append(prebuild.plan_for(name, dims))
+        finally:
+            os.environ.pop('FLEX_RNN_TILE') if old is None else os.environ.__setitem__('FLEX_RNN_TILE', old)
     for name, dims in NO_ALLOC_DIMS:
         plans.append(prebuild.plan_for(name, dims, tile=no_alloc_tile(name, dims)))
     for name, dims in OTHER:
