@@ -497,6 +497,9 @@ class Emitter:
         """Occupancy request of the row kernels (`TileConfig.WPE` waves per SIMD): the compiler then fits the
         kernel into 512 / WPE registers instead of using all a workgroup of its size may have."""
         wpe = int(getattr(self.tile, 'WPE', 0) or 0)
+        wn = int(getattr(self.tile, 'WN', 0) or 0)
+        if not wpe and wn:          # a lower bound only: 512 / WN registers as budget, more waves if fewer are used
+            return f' __attribute__((amdgpu_waves_per_eu({wn})))'
         return f' __attribute__((amdgpu_waves_per_eu({wpe},{wpe})))' if wpe else ''
 
     def _lane_prolog(self) -> str:

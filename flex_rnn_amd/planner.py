@@ -86,6 +86,9 @@ class TileConfig:
     MS: int = 1          # instances sharing the rows of one (batch, head, chunk) in the gradient kernel;
                          # above 1 the row/scalar-input grads are summed across them with atomics
     WPE: int = 0         # waves per SIMD the row kernels are compiled for (0 = whatever the compiler arrives at)
+    WN: int = 0          # row kernels: at least this many waves per SIMD (0 = no request).  A workgroup of four waves may use a
+                         # SIMD's whole register file; near 256 registers the compiler then parks values in the accumulation
+                         # registers or in scratch, with 2 here it allocates within 256 (Mamba-1's reverse scan: 0.33 -> 0.31 ms)
     UR: int = 2          # row kernels: unrolling of the loop over the staged timesteps
     NB: int = 1          # row sums leave a step without a branch (every lane of a group stores them): bit 0 = forward
                          # kernel, bit 1 = reverse scan.  Lets the compiler overlap consecutive steps, at the price of registers.
