@@ -277,6 +277,8 @@ def check_tile(tile: TileConfig, H: int, N: int, part: Partition) -> None:
     for k in ('L', 'C', 'R', 'W', 'DT', 'TS'):
         assert getattr(t, k) >= 1 and _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be a power of two'
     assert t.HB >= 1 and 1 <= t.MS <= 65535, 'HB and MS must be positive (MS is a grid dimension)'
+    assert 0 <= t.WPE <= 8 and 0 <= t.WN <= 8, 'WPE and WN are waves per SIMD (0 = no request, at most 8)'
+    assert t.UR >= 1 and 0 <= t.NB <= 3 and t.DF in (0, 1) and t.SH in (0, 1), 'UR >= 1, NB in 0..3, DF and SH 0 or 1'
     for k in ('R1', 'W1'):
         assert getattr(t, k) == 0 or _is_pow2(getattr(t, k)), f'tile field {k}={getattr(t, k)} must be 0 or a power of two'
     assert t.L <= 64 and t.L * t.C == N, f'tile covers {t.L}*{t.C} columns, the state has {N}'

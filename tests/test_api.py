@@ -225,6 +225,13 @@ def test_row_kernel_candidate_tiles_are_valid():
             for v in variants:
                 planner.check_tile(v, plan.H, plan.NP, plan.part)
     assert (8, 16, 2, 8) in launch.row_kernel_tiles(prebuild.plan_for('rwkv7'), False)
+    # large problems also time the first tile with a register budget of half a SIMD's file; knob values out of range are refused
+    plan = prebuild.plan_for('rwkv7')
+    assert any(v.WN == 2 for v in launch.row_kernel_variants(plan, False)) and all(v.WN == 0 for v in launch.row_kernel_variants(
+        prebuild.plan_for('rwkv7', (2, 64, 2, 128, 128)), False))
+    for bad in (dict(WN=9), dict(DF=2), dict(NB=4), dict(UR=0)):
+        with pytest.raises(AssertionError):
+            planner.check_tile(dataclasses.replace(plan.tile, **bad), plan.H, plan.NP, plan.part)
 
 
 def test_timed_picks_are_kept_beside_the_cache(tmp_path, monkeypatch):
