@@ -102,6 +102,33 @@ class jit:
                 fwd = self.forward_func
             return fwd.forward_only(inputs, state)
 
+    def segmented(self, *args, segment: int):
+        """The results (and gradients) of a call, computed `segment` timesteps at a time under activation
+        checkpointing (an addition to the reference's interface, for sequences whose hidden buffers do not fit):
+        only the states at the segment boundaries are kept for the backward pass, which runs a segment's forward
+        kernel again just before that segment's backward kernels.  The hidden buffers - fp32 state and d-state
+        checkpoints every 16 timesteps, saved row sums - then exist for one segment at a time instead of the whole
+        sequence, at the price of one more forward pass.  Segments are planned like calls of a `dynamic` instance."""
+        from torch.utils.checkpoint import checkpoint
+        inputs, state = split_list(args, [self.ninputs, self.nstates])
+        assert segment >= 1
+        T = max(i.shape[1] for i in inputs)
+        if getattr(self, '_segments', None) is None:
+            self._segments = self if self.is_dynamic else jit(self.step, self.ninputs + self.nstates, dynamic=True)
+        outs = [[] for _ in range(self.noutputs)]
+        for t0 in range(0, T, segment):
+            part = [x[:, t0:t0 + segment] if x.shape[1] != 1 else x for x in inputs]
+            if isinstance(self._segments, jit) and part[0].is_cuda and not isinstance(part[0], th._subclasses.FakeTensor):
+                # (plans are traced with torch.func, which refuses to run under the saved-tensor hooks of `checkpoint`)
+                self._segments._entry(part, list(state), dry=False)
+            res = checkpoint(self._segments.apply, *part, *state, use_reentrant=False)
+            for k in range(self.noutputs):
+                outs[k].append(res[k])
+            state = tuple(res[self.noutputs:])
+        if T == 0:
+            return self._segments.apply(*args)
+        return (*[th.cat(o, dim=1) for o in outs], *state)
+
     # ------------------------------------------------------------------ plain per-timestep loop
     def naive(self, *args, dtype=th.float32):
         """Pure-PyTorch per-timestep loop with the compiled path's calling convention

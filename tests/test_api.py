@@ -267,3 +267,23 @@ def test_compiled_plan_keeps_its_host_interface():
     for m in ('_launch', '_tune', '_select', '_register', '_install', '_row_builds', 'forward', 'forward_only', 'backward',
               'static_layout', 'launch_static'):
         assert callable(getattr(CompiledPlan, m, None)), m
+
+
+def test_segmented_call_slices_time_and_carries_the_state():
+    """`jit.segmented` (the compiled operator replaced by the plain loop here, which takes the same arguments): outputs,
+    final states and all gradients equal those of one call over the whole sequence; time-independent inputs are not
+    sliced; the last segment may be shorter."""
+    step, xs, ss = cases.make_inputs('mamba', 2, 11, 2, 4, 4, dtype=th.float64)
+    f = flex_rnn_amd.jit(step)
+    f._segments = type('Loop', (), {'apply': staticmethod(lambda *a: f.naive(*a, dtype=th.float64))})()
+    xg = [x.clone().requires_grad_() for x in xs]
+    sg = [s.clone().requires_grad_() for s in ss]
+    whole = f.naive(*xg, *sg, dtype=th.float64)
+    gy = [th.randn_like(r) for r in whole]
+    want = th.autograd.grad(whole, xg + sg, gy)
+    for segment in (4, 11, 16, 1):
+        got = f.segmented(*xg, *sg, segment=segment)
+        assert all(a.shape == b.shape for a, b in zip(got, whole))
+        assert all(th.allclose(a, b, rtol=0, atol=1e-12) for a, b in zip(got, whole)), segment
+        grads = th.autograd.grad(got, xg + sg, gy)
+        assert all(th.allclose(a, b, rtol=0, atol=1e-10) for a, b in zip(grads, want)), segment

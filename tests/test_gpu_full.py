@@ -236,6 +236,23 @@ def test_row_kernel_knobs_against_oracle(name, dims, knobs, monkeypatch):
     assert all(getattr(tile, k) == int(v) for k, v in (kv.split('=') for kv in knobs.split(',')))
 
 
+@pytest.mark.parametrize('name,dims', warm.SEGMENTED_CASES)
+def test_segmented_call_against_oracle(name, dims):
+    """`jit.segmented` (32 timesteps at a time under activation checkpointing, a shorter last segment): outputs, final
+    state and all gradients against the oracle's single pass over the whole sequence."""
+    print(f'case segmented {name} {dims}', flush=True)
+    wl = configs.make(name, dims=dims)
+    dy, dS = configs.upstream_grads(wl)
+    want = recurrence.loop_with_grads(wl.step, wl.inputs, wl.states, dy, dS, dtype=th.float64)
+    want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
+    f = flex_rnn_amd.jit(wl.step)
+    xg = [x.requires_grad_() for x in _gpu(wl.inputs)]
+    sg = [s.requires_grad_() for s in _gpu(wl.states)]
+    res = f.segmented(*xg, *sg, segment=warm.SEGMENT)
+    grads = th.autograd.grad(res, xg + sg, grad_outputs=[g.cuda().to(r.dtype) for g, r in zip(dy + dS, res)])
+    recurrence.assert_all_close(list(res) + list(grads), want, TOL[wl.dtype], f'segmented {name}')
+
+
 @pytest.mark.parametrize('name', ['rwkv7', 'mamba1', 'mamba2'])
 def test_infer_matches_call(name):
     """`jit.infer` (no checkpoints, no saved sums) returns what a normal call returns."""

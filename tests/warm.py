@@ -51,6 +51,11 @@ def no_alloc_tile(name, dims):
 KNOB_CASES = [('rwkv7', (2, 37, 2, 64, 64), 'DF=1,NB=3,UR=4'), ('mamba1', (2, 45, 4, 128, 16), 'DF=1,NB=3')]
 
 
+# tests/test_gpu_full.py::test_segmented_call_against_oracle: sequences walked SEGMENT timesteps at a time
+SEGMENT = 32
+SEGMENTED_CASES = [('gated_delta_rule', (2, 77, 2, 128, 128)), ('mamba1', (2, 45, 4, 128, 16))]
+
+
 EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
 
 
@@ -93,6 +98,9 @@ def warm(force=False, seen=None):
             plans.append(prebuild.plan_for(name, dims))
         finally:
             os.environ.pop('FLEX_RNN_TILE') if old is None else os.environ.__setitem__('FLEX_RNN_TILE', old)
+    for name, (B, T, H, M, N) in SEGMENTED_CASES:
+        for seg in sorted({min(SEGMENT, T), T % SEGMENT} - {0}):
+            plans.append(prebuild.plan_for(name, (B, seg, H, M, N)))
     for name, dims in NO_ALLOC_DIMS:
         plans.append(prebuild.plan_for(name, dims, tile=no_alloc_tile(name, dims)))
     for name, dims in OTHER:
