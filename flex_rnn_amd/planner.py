@@ -195,7 +195,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
             R_ //= 2
 
         def waves_per_wg(r):
-            return max(1, min(4, M // (G_ * r))) if G_ * r <= M else 1
+            return _pow2_floor(max(1, min(4, M // (G_ * r)))) if G_ * r <= M else 1      # (a power of two; the grid covers ragged rows)
 
         def total_waves(r):
             w = waves_per_wg(r)
@@ -233,7 +233,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
         # lane there, and a chunk short enough for 64 registers of history per state (measured:
         # anything more drops the kernel to one wave per SIMD or spills)
         R1 = 1
-        W1 = max(1, min(4, M // G)) if G <= M else 1
+        W1 = _pow2_floor(max(1, min(4, M // G))) if G <= M else 1
         DT = max(2, min(16, _pow2_floor(64 // max(C * part.nstates, 1))))
     else:
         DT = 16

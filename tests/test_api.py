@@ -234,6 +234,18 @@ def test_row_kernel_candidate_tiles_are_valid():
             planner.check_tile(dataclasses.replace(plan.tile, **bad), plan.H, plan.NP, plan.part)
 
 
+def test_tile_heuristic_gives_valid_tiles_for_ragged_shapes():
+    """Row counts and widths that are not powers of two, single rows, narrow and wide states: the heuristic's tile
+    passes the planner's own check (a row count of 24 once gave three waves per workgroup)."""
+    from flex_rnn_amd import prebuild
+    for name in ('mamba1', 'mamba2', 'rwkv7', 'gated_delta_rule', 'delta_rule'):
+        for M in (1, 3, 24, 40, 100, 192):
+            for N in ((8, 16) if name == 'mamba1' else (16, 48, 128)):
+                for B, T, H in ((1, 19, 1), (8, 1024, 32)):
+                    plan = prebuild.plan_for(name, (B, T, H, M, N))
+                    planner.check_tile(plan.tile, plan.H, plan.NP, plan.part)
+
+
 def test_timed_picks_are_kept_beside_the_cache(tmp_path, monkeypatch):
     """The choice among candidate builds is stored per (kernel, candidates, device, B, H, M) - not per
     sequence length - and found again by a fresh process (here: a fresh `_Picks`)."""

@@ -30,6 +30,9 @@ RUNS = [
     ('hgrn', '2,8,1,64,1', 'f32', 1),               # vector state (N = 1)
     ('rwkv4', '2,8,1,32,1', 'f32', 0),              # three states, comparisons
     ('mlstm_gates', '2,8,2,16,1', 'f32', 1),        # three outputs
+    # row counts that are not a power of two (the heuristic once asked for three waves per workgroup there)
+    ('cfg:mamba1', '2,35,4,24,16', 'bf16', 1),
+    ('cfg:rwkv7', '2,17,2,48,64', 'f32', 0),
     # sequence lengths that are not a multiple of the chunk (partial last chunk), and T = 1
     ('cfg:rwkv7', '1,37,1,128,128', 'f32', 0),
     ('cfg:mamba1', '2,13,2,128,16', 'f32', 1),
