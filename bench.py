@@ -184,8 +184,8 @@ def measure(name, steps, warmup, traffic_records):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
-    ap.add_argument('--steps', type=int, default=20)
-    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--steps', type=int, default=100)
+    ap.add_argument('--warmup', type=int, default=20)
     ap.add_argument('--workload', default='rwkv7', choices=sorted(WORK))
     ap.add_argument('--no-cpu', action='store_true', help='skip the CPU baseline leg')
     ap.add_argument('--no-others', action='store_true', help='skip the short runs of the other three GPU workloads')
@@ -217,7 +217,7 @@ def main():
     if name == 'rwkv7' and not args.no_others:
         others = {}
         for other in ('mamba1', 'mamba2', 'gated_delta_rule'):
-            n_steps, n_warm = (10, 3) if other == 'gated_delta_rule' else (20, 10)     # (short steps: long enough for the clocks to settle)
+            n_steps, n_warm = (20, 5) if other == 'gated_delta_rule' else (50, 20)     # (short steps: long enough for the clocks to settle)
             r = measure(other, n_steps, n_warm, traffic_records)
             rf = r['roofline']
             others[other] = {'workload': r['config']['workload'], 'ms_per_step': r['ms_per_step'], 'tokens_per_s': r['value'],
