@@ -263,6 +263,11 @@ class _Picks:
             h.update(runtime.source_key(spec.name, spec.source).encode())
         return f'{name}|{h.hexdigest()[:20]}|{device_name}|B{plan.B}H{plan.H}M{plan.M}'
 
+    # choices for the benchmark workloads as timed on an MI355X, shipped with the package: a fresh cache directory then
+    # starts from them (they apply as long as the candidate sources and the device name are the ones they were timed
+    # with; anything else is timed as usual).  Written by `export_shipped_picks`.
+    SHIPPED = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'picks_mi355x.json')
+
     def _path(self):
         return os.path.join(runtime.cache_dir(), 'picks.json')
 
@@ -270,13 +275,14 @@ class _Picks:
         path = self._path()
         if self.loaded_from != path:            # (the cache directory may be redirected between plans, e.g. by tests)
             self.loaded_from = path
-            try:
-                with open(path) as f:
-                    disk = json.load(f)
-                for k, v in disk.items():
-                    self.mem.setdefault(k, v)
-            except (OSError, ValueError):
-                pass
+            for src in (path, self.SHIPPED):    # (what this machine timed itself comes first)
+                try:
+                    with open(src) as f:
+                        disk = json.load(f)
+                    for k, v in disk.items():
+                        self.mem.setdefault(k, v)
+                except (OSError, ValueError):
+                    pass
 
     def get(self, key, n):
         with self.lock:
@@ -308,6 +314,36 @@ class _Picks:
 
 
 PICKS = _Picks()
+
+
+def shipped_pick_keys(device_name: str, names=('rwkv7', 'mamba1', 'mamba2', 'gated_delta_rule')):
+    """{key: number of candidates} of the kernels of the benchmark workloads at their full sizes, for the current
+    kernel sources (nothing is compiled)."""
+    from . import prebuild
+    out = {}
+    for wl in names:
+        plan = prebuild.plan_for(wl)
+        sets = {'frnn_fw': row_kernel_specs(plan, False), 'frnn_bw1': row_kernel_specs(plan, True),
+                'frnn_fwi': row_kernel_specs(plan, False, save=False)}
+        for kname, specs in sets.items():
+            out[PICKS.key(kname, [(s_, None, None) for s_ in specs], device_name, plan)] = len(specs)
+        if needs_gradient_kernel(plan.part):
+            builds = gradient_kernel_builds(plan)
+            out[PICKS.key('frnn_bw2', builds, device_name, plan)] = len(builds)
+    return out
+
+
+def export_shipped_picks(device_name: str, path: str = None) -> int:
+    """Writes the choices this machine's cache holds for the benchmark workloads (current kernel sources, device
+    `device_name`) to the package's shipped file; returns how many were found."""
+    with PICKS.lock:
+        PICKS.loaded_from = None
+        PICKS._load()
+        have = {k: PICKS.mem[k] for k, n in shipped_pick_keys(device_name).items()
+                if k in PICKS.mem and 0 <= PICKS.mem[k].get('index', -1) < n}
+    with open(path or PICKS.SHIPPED, 'w') as f:
+        json.dump(have, f, indent=0, sort_keys=True)
+    return len(have)
 
 
 class CompiledPlan:

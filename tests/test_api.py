@@ -299,3 +299,35 @@ def test_segmented_call_slices_time_and_carries_the_state():
         assert all(th.allclose(a, b, rtol=0, atol=1e-12) for a, b in zip(got, whole)), segment
         grads = th.autograd.grad(got, xg + sg, gy)
         assert all(th.allclose(a, b, rtol=0, atol=1e-10) for a, b in zip(grads, want)), segment
+
+
+def test_shipped_picks_are_well_formed_and_name_existing_candidates():
+    """The timed choices shipped for the benchmark workloads: one record per key with an index into the candidate list
+    and one timing per candidate; those whose key matches the current row-kernel sources index an existing candidate
+    (a key for other sources is ignored at run time and the kernel is timed again)."""
+    import json
+    from flex_rnn_amd import launch, prebuild
+    shipped = json.load(open(launch.PICKS.SHIPPED))
+    assert shipped and all(isinstance(v['index'], int) and 0 <= v['index'] < max(len(v['ms']), 1) for v in shipped.values())
+    devices = {k.split('|')[2] for k in shipped}
+    matched = 0
+    for dev in devices:
+        for wl in ('rwkv7', 'mamba1'):
+            plan = prebuild.plan_for(wl)
+            for kname, specs in (('frnn_fw', launch.row_kernel_specs(plan, False)), ('frnn_bw1', launch.row_kernel_specs(plan, True))):
+                key = launch.PICKS.key(kname, [(s, None, None) for s in specs], dev, plan)
+                if key in shipped:
+                    matched += 1
+                    assert shipped[key]['index'] < len(specs) == len(shipped[key]['ms'])
+    # a cache directory without choices of its own starts from the shipped ones
+    import os, tempfile
+    old = os.environ.get('FLEX_RNN_CACHE')
+    with tempfile.TemporaryDirectory() as tmp:
+        os.environ['FLEX_RNN_CACHE'] = tmp
+        try:
+            key = next(iter(shipped))
+            assert launch._Picks().get(key, len(shipped[key]['ms']))['index'] == shipped[key]['index']
+        finally:
+            os.environ.pop('FLEX_RNN_CACHE') if old is None else os.environ.__setitem__('FLEX_RNN_CACHE', old)
+    if not matched:
+        pytest.skip('the shipped choices were timed on other kernel sources; they are ignored until exported again')
