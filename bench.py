@@ -169,13 +169,15 @@ def measure(name, steps, warmup, traffic_records):
 
     res['row_kernel_builds'] = {k: {'candidates (L, C, R, W, branch-free sums, unroll, deferred flush, min waves per SIMD)':
                                     [knobs(t_, k == 'frnn_bw1') for t_ in launch.row_kernel_variants(compiled.plan, k == 'frnn_bw1')],
-                                    'ms': compiled.build_times.get(k) and [finite(v) for v in compiled.build_times[k]]}
+                                    'ms': compiled.build_times.get(k) and [finite(v) for v in compiled.build_times[k]],
+                                    'ms_source': compiled.build_source.get(k, 'not timed: one candidate, or timing switched off')}
                                 for k in ('frnn_fw', 'frnn_bw1')}
     bt = compiled.bw2_times
-    res['gradient_kernel_builds'] = [
-        {'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
-         'ms': finite(bt[i]) if bt and i < len(bt) else None}
-        for i, (_, _, r) in enumerate(compiled.bw2_builds)]
+    res['gradient_kernel_builds'] = {
+        'ms_source': compiled.build_source.get('frnn_bw2', 'not timed: one candidate, or timing switched off'),
+        'candidates': [{'vgprs': r and r['vgprs'], 'waves_per_simd': r and r['occupancy'], 'spill_bytes': r and r['scratch'],
+                        'ms': finite(bt[i]) if bt and i < len(bt) else None}
+                       for i, (_, _, r) in enumerate(compiled.bw2_builds)]}
     del xs, ss, gy, f
     th.cuda.empty_cache()
     return res

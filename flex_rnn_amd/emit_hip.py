@@ -25,7 +25,7 @@ from __future__ import annotations
 
 import math
 import os
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import List, Sequence, Tuple
 
 import torch as th
@@ -238,6 +238,8 @@ class KernelSpec:
     tensors: List[str]          # logical tensor names, in Args order
     block: int
     grid: Tuple[str, str, str]  # python expressions over B, T, H, M, nch
+    geom: dict = field(default_factory=dict)    # what the grid is meant to cover (rows per workgroup, chunks per workgroup, row slices):
+                                # the host checks the evaluated grid against it before a launch when asked to
 
 
 class _Args:
@@ -660,14 +662,16 @@ class Emitter:
             out.append(f'{ind}  }} }}\n')
             return out
 
-        if not df:
+        ck_late = df
+        if not ck_late:
             body += checkpoint()
         body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
         body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
-        if df:
+        if ck_late:
             body += checkpoint()
+        if df:
             if nout or naux:        # the chunk before this one (always a whole one)
                 body.append(f'    if (t0 > 0) {{\n')
                 body += flush(f't0 - {TS}', str(TS), f'((t0 / {TS}) & 1) ^ 1', '      ')
@@ -743,7 +747,7 @@ class Emitter:
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){self._row_attr()} {kname}(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
         source = PRELUDE + A.struct() + self._row_macros() + fn_src + '\n' + kernel
-        return KernelSpec(kname, source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
+        return KernelSpec(kname, source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'), {'kind': 'row', 'MT': MT})
 
     # ------------------------------------------------------------------ bw1
     def bw1(self) -> KernelSpec:
@@ -869,7 +873,8 @@ class Emitter:
             out.append(f'{ind}  }} }}\n')
             return out
 
-        if not df:
+        ck_late = df
+        if not ck_late:
             body += d_checkpoint()
         body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
@@ -880,8 +885,9 @@ class Emitter:
                         f'#pragma unroll\n    for (int c = 0; c < {cc}; c++) Sh{k}_0[r][c] = pS{k}[r][c];\n')
         body.append(f'    if (t0 >= {TS}) {{\n' + stg.load(f't0 - {TS}', '      ')
                     + ''.join(ckpt_fetch(k, f't0 / {DT} - 1', '      ') for k in range(nst if needs_state else 0)) + '    }\n')
-        if df:
+        if ck_late:
             body += d_checkpoint()
+        if df:
             pre = flush(f't0 + {TS}', f'min({TS}, T - (t0 + {TS}))' if tail else str(TS), f'((t0 / {TS}) & 1) ^ 1', '      ')
             if pre:                 # the chunk walked before this one (the later timesteps; only that one can be partial)
                 body.append('    if (t0 < tlast) {\n')
@@ -1034,7 +1040,7 @@ class Emitter:
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){self._row_attr()} frnn_bw1(Args A) {{\n'
                   + ''.join(src) + ''.join(body) + '}\n')
         source = PRELUDE + A.struct() + self._row_macros() + '\n'.join(fns) + '\n' + kernel
-        return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'))
+        return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'), {'kind': 'row', 'MT': MT})
 
     # ------------------------------------------------------------------ bw2
     def bw2(self, waves_per_simd: int = 0, prefetch: int = 4) -> KernelSpec:
@@ -1523,4 +1529,6 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
         kernel = (f'extern "C" __global__ void __launch_bounds__({NT}){attr} frnn_bw2(Args A) {{\n' + ''.join(b) + '}\n')
         source = PRELUDE + A.struct() + helper + re_src + '\n' + drow_src + '\n' + epi_src + '\n' + pre_src + '\n' + kernel
         gx, gy, gz = f'(nch + {cpb - 1}) // {cpb}', f'B * (H // {HB})', str(MS // IPB if share else MS)
-        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'({gx}) * {gy}', '1', gz) if fold else (gx, gy, gz))
+        geom = {'kind': 'grad', 'cpb': cpb, 'HB': HB, 'gz': int(gz), 'fold': fold,
+                'rows_per_z': plan.M if MS == 1 else (MR * IPB if share else MR)}
+        return KernelSpec('frnn_bw2', source, list(A.names), NT, (f'({gx}) * {gy}', '1', gz) if fold else (gx, gy, gz), geom)

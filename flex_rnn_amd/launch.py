@@ -37,6 +37,7 @@ def kernel_specs(plan, prefetch: int = 4) -> List[KernelSpec]:
 
 
 _seen_lock = threading.Lock()
+_CHECK = os.environ.get('FLEX_RNN_CHECK', '0') == '1'      # audit every launch (`CompiledPlan._audit`)
 MAX_SPILL_BYTES = 64      # per lane; the untimed choice among gradient-kernel builds does not accept more
 
 
@@ -117,12 +118,37 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
         top = ranked[0][0].source
         wps = int(top.split('amdgpu_waves_per_eu(')[1].split(',')[0]) if 'amdgpu_waves_per_eu(' in top else 0
         first = len(cands)
-        for alt in (ms // 4, ms * 4):
-            if alt >= 2 and -(-plan.M // alt) >= 4 and alt <= 65535:
-                em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
-                add([em_alt.bw2(waves_per_simd=wps, prefetch=4)], optional=True)
+        for alt in _alt_splits(plan):
+            em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
+            add([em_alt.bw2(waves_per_simd=wps, prefetch=4)], optional=True)
         ranked += cands[first:]
     return ranked
+
+
+def gradient_kernel_specs(plan, waves_per_simd: int = 0):
+    """The candidate sources of the gradient kernel that do not depend on a compiler report: 4 and 2 checkpoint rows
+    in flight and, with split rows, a quarter and four times as many splits (what `gradient_kernel_builds` makes,
+    less the occupancy requests).  Nothing is compiled."""
+    em = Emitter(plan)
+    specs = [em.bw2(prefetch=pd) for pd in (4, 2)]
+    for alt in _alt_splits(plan):
+        em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
+        specs.append(em_alt.bw2(waves_per_simd=waves_per_simd, prefetch=4))
+    out, seen_src = [], set()
+    for sp in specs:
+        if sp.source not in seen_src:
+            seen_src.add(sp.source)
+            out.append(sp)
+    return out
+
+
+def _alt_splits(plan):
+    """Other row-split counts of the gradient kernel that are worth timing: a quarter and four times the plan's own
+    (every build accumulates atomically into the same fp32 buffers, so they are interchangeable at run time)."""
+    ms = plan.tile.MS
+    if ms <= 1:
+        return []
+    return [alt for alt in (ms // 4, ms * 4) if alt >= 2 and -(-plan.M // alt) >= 4 and alt <= 65535]
 
 
 def row_kernel_tiles(plan, reverse: bool):
@@ -176,6 +202,11 @@ def row_kernel_variants(plan, reverse: bool):
     bit = 2 if reverse else 1
     base = plan.tile
     big = plan.B * plan.T * plan.H * plan.M * plan.NP >= TUNE_KNOBS_FROM
+    # A sequence with a partial last staging block gets no deferred-flush candidate: the one GPU memory fault on
+    # record involved that form on such a sequence, and no cause has been shown (an explicit override still builds it,
+    # for the CPU harness)
+    ts = base.DT if (reverse and plan.part.dstep_needs_state) else base.TS
+    may_defer = plan.T % ts == 0
     out = []
     for k, (L, C, r, w) in enumerate(row_kernel_tiles(plan, reverse)):
         tile = dataclasses.replace(base, L=L, C=C)
@@ -183,8 +214,9 @@ def row_kernel_variants(plan, reverse: bool):
         own = (base.NB, base.DF, base.UR, base.WN)      # (the plan's own setting first)
         knobs = [own]
         if big:
-            knobs += [(base.NB ^ bit, base.DF, base.UR, base.WN), (base.NB, base.DF ^ 1, base.UR, base.WN),
-                      (base.NB ^ bit, base.DF ^ 1, base.UR, base.WN)]
+            knobs += [(base.NB ^ bit, base.DF, base.UR, base.WN)]
+            if may_defer or base.DF:
+                knobs += [(base.NB, base.DF ^ 1, base.UR, base.WN), (base.NB ^ bit, base.DF ^ 1, base.UR, base.WN)]
             if k == 0 and not (reverse and plan.part.dstep_needs_state):
                 knobs.append((base.NB | bit, base.DF, 4, base.WN))
             if k == 0 and not base.WN and not base.WPE:
@@ -248,8 +280,11 @@ class _Picks:
     batch, heads, rows) in memory and in `picks.json` beside the cached code objects, so that the choice -
     and with it the order of the additions inside every reduction - is made once and then repeats: later
     plans and later processes run the same build without timing anything.  The sequence length is not
-    part of the key: it changes how long a kernel runs, not which candidate is fastest, and calls over
-    pieces of a sequence then run the same code as one call over the whole."""
+    part of the key: it changes how long a kernel runs, not which candidate is fastest.  It does enter
+    through the candidate set, though: whether the length is a multiple of the staging depth is baked into the
+    sources, and the code-generation knobs only become candidates from `TUNE_KNOBS_FROM` state-element timesteps,
+    so calls over pieces of a sequence run the same build as one call over the whole only when both lengths are
+    aligned and on the same side of that threshold."""
 
     def __init__(self):
         self.lock = threading.Lock()
@@ -348,6 +383,7 @@ def export_shipped_picks(device_name: str, path: str = None) -> int:
 
 class CompiledPlan:
     _tune_pending = frozenset()
+    _tune_rounds = 4            # rounds over the candidates when a kernel is timed; the first one is not counted
 
     def __init__(self, plan, state_meta=None, device=None):
         self.plan = plan
@@ -376,6 +412,7 @@ class CompiledPlan:
 
         self._load = load
         self.builds, self.build_times, self._grid, self._packer = {}, {}, {}, {}
+        self.build_source = {}      # kernel -> 'timed in this process' | 'stored choice' (where `build_times` come from)
         if plan.B == 0 or plan.T == 0:
             return                          # nothing will ever be launched for an empty batch or no timesteps
         # Every kernel comes in a few candidate builds (tiles and code-generation knobs of the row kernels; prefetch
@@ -424,6 +461,7 @@ class CompiledPlan:
             self.builds[name] = [(s_, self._load(s_, p_) if p_ is not None else None, r_) for s_, p_, r_ in built]
         if chosen is not None:
             self.build_times[name] = [float('inf') if t is None else t for t in chosen.get('ms', [])] or None
+            self.build_source[name] = 'stored choice'
             self._select(name, chosen['index'])
             return
         if len(built) > 1 and self._tune_on and name not in self._fixed:
@@ -457,15 +495,74 @@ class CompiledPlan:
         self._packer[name] = struct.Struct('<' + 'q5q' * max(len(spec.tensors), 1) + '5q')
 
     # ------------------------------------------------------------------ launch helper
-    def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
+    _on_gpu = True          # (the CPU harness of the tests runs the same host code on CPU tensors)
+
+    def _expected(self, name: str):
+        """(shape, dtype, must be contiguous?) the kernels assume for the tensor called `name` in a kernel's
+        argument list."""
+        pl, p = self.plan, self.plan.part
+        B, T, H, M, N = pl.B, pl.T, pl.H, pl.M, pl.N
+        kind = name.rstrip('0123456789')
+        k = int(name[len(kind):]) if len(name) > len(kind) else 0
+        if kind in ('in', 'din'):
+            bc, cls = pl.in_bcast[k], pl.in_cls[k]
+            shape = (1 if bc[0] else B, 1 if bc[1] else T, 1 if bc[2] else H,
+                     M if cls in ('col', 'mat') else 1, N if cls in ('row', 'mat') else 1)
+            dtype = th.float32 if (kind == 'din' and k in set(pl.atomic)) else pl.in_dtypes[k]
+            return shape, dtype, False
+        if kind in ('st', 'stT', 'dst', 'dstT'):
+            return (B, H, M, N), pl.st_dtypes[k], False
+        if kind in ('sck', 'dck'):
+            return (B, H, pl.nchunks, M, pl.NP), th.float32, True
+        if kind in ('out', 'dout'):
+            return (B, T, H, M), pl.out_dtypes[k], False
+        if kind == 'aux':
+            return (len(p.aux), B, H, T, M), th.float32, True
+        if kind == 'daux':
+            return (len(p.daux), B, H, T, M), th.float32, True
+        raise AssertionError(f'unknown kernel tensor {name}')
+
+    def _audit(self, kname: str, tensors: Dict[str, th.Tensor]):
+        """Checks, before a launch, what the kernel takes on trust: every tensor has the shape and element type its
+        index arithmetic was emitted for, its last addressed element (offset + sum of (extent - 1) * stride) lies inside
+        its storage, hidden buffers are contiguous, and the grid covers the rows / chunks / (batch, head) pairs of the
+        plan exactly once.  On with FLEX_RNN_CHECK=1 (the tests switch it on); costs some tens of microseconds per launch."""
+        spec, _ = self.kernels[kname]
+        pl = self.plan
+        for name in spec.tensors:
+            t = tensors[name]
+            shape, dtype, contig = self._expected(name)
+            assert tuple(t.shape) == tuple(shape), f'{kname}: tensor {name} has shape {tuple(t.shape)}, the kernel indexes {tuple(shape)}'
+            assert t.dtype == dtype, f'{kname}: tensor {name} is {t.dtype}, the kernel was emitted for {dtype}'
+            assert not contig or t.is_contiguous(), f'{kname}: hidden buffer {name} must be contiguous'
+            if t.numel():
+                assert all(st >= 0 for st in t.stride()), f'{kname}: tensor {name} has a negative stride'
+                last = t.storage_offset() + sum((n - 1) * st for n, st in zip(t.shape, t.stride()))
+                room = t.untyped_storage().nbytes() // t.element_size()
+                assert last < room, f'{kname}: tensor {name} reaches element {last} of a storage that holds {room}'
+        g, geo = self._grid[kname], spec.geom
+        assert all(1 <= v for v in g) and g[0] < 2 ** 31 and g[1] <= 65535 and g[2] <= 65535, f'{kname}: grid {g} is not launchable'
+        if geo.get('kind') == 'row':
+            MT = geo['MT']
+            assert g == (-(-pl.M // MT), pl.H, pl.B), f'{kname}: grid {g} does not cover {pl.M} rows in tiles of {MT} x {pl.H} heads x batch {pl.B}'
+        elif geo.get('kind') == 'grad':
+            gx, gy = -(-pl.nchunks // geo['cpb']), pl.B * (pl.H // geo['HB'])
+            want = (gx * gy, 1, geo['gz']) if geo['fold'] else (gx, gy, geo['gz'])
+            assert g == want, f'{kname}: grid {g}, expected {want}'
+            assert geo['gz'] * geo['rows_per_z'] >= pl.M, f'{kname}: {geo["gz"]} row slices of {geo["rows_per_z"]} do not cover {pl.M} rows'
+
+    def _pack(self, kname: str, tensors: Dict[str, th.Tensor]):
+        """(argument block, device) of a launch of kernel `kname` on `tensors`."""
         spec, kern = self.kernels[kname]
         pl = self.plan
         vals = []
         dev = None
         for name in spec.tensors:
+            if name not in tensors:
+                raise AssertionError(f'kernel {kname} takes a tensor called {name}; the call passed {sorted(tensors)}')
             t = tensors[name]
             if t.device != dev:
-                assert t.is_cuda, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
+                assert t.is_cuda or not self._on_gpu, f'{name}: the compiled path runs on the GPU only (got a {t.device} tensor)'
                 assert dev is None, 'all tensors must live on the same device'
                 assert self.device is None or t.device == self.device, \
                     f'this instance was compiled for {self.device}; got a tensor on {t.device}'
@@ -474,7 +571,13 @@ class CompiledPlan:
             vals.extend(_strides5(t))
         if not spec.tensors:
             vals = [0] * 6
-        buf = self._packer[kname].pack(*vals, pl.B, pl.T, pl.H, pl.M, pl.nchunks)
+        if _CHECK:
+            self._audit(kname, tensors)
+        return self._packer[kname].pack(*vals, pl.B, pl.T, pl.H, pl.M, pl.nchunks), dev
+
+    def _launch(self, kname: str, tensors: Dict[str, th.Tensor]):
+        spec, kern = self.kernels[kname]
+        buf, dev = self._pack(kname, tensors)
         grid = self._grid[kname]
         other = dev is not None and th.cuda.current_device() != dev.index
         with (th.cuda.device(dev) if other or dev is None else contextlib.nullcontext()):
@@ -487,6 +590,18 @@ class CompiledPlan:
                 self.profile_events.append((kname, e0, e1))
             else:
                 kern.launch(grid, (spec.block, 1, 1), buf, stream=stream)
+
+    def _timed_launch(self, kname: str, tensors) -> float:
+        """One launch of the selected build of `kname`, waited for; milliseconds."""
+        e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
+        e0.record()
+        self._launch(kname, tensors)
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1)
+
+    def _capturing(self) -> bool:
+        return th.cuda.is_current_stream_capturing()
 
     # ------------------------------------------------------------------ hidden buffers in the library's scratch
     def static_layout(self):
@@ -522,6 +637,7 @@ class CompiledPlan:
                 slots.append((48 * j, off, n, 1 if name in clear else 0))
                 vals.extend([0] * 6)
                 continue
+            assert name in tensors, f'kernel {kname} takes a tensor called {name} that is neither in the static layout nor passed by the caller'
             t = tensors[name]
             assert t.is_cuda and (dev is None or t.device == dev), 'all tensors must live on one GPU'
             dev = t.device
@@ -539,7 +655,7 @@ class CompiledPlan:
         fastest.  The kernels only store and
         accumulate; `accumulators` (what they add into) are put back afterwards.  Synchronises,
         once per kernel and plan; skipped while the stream is being captured."""
-        if name not in self._tune_pending or th.cuda.is_current_stream_capturing():
+        if name not in self._tune_pending or self._capturing():
             return
         self._tune_pending.discard(name)
         n = len(self.builds[name])
@@ -548,25 +664,22 @@ class CompiledPlan:
         if rec is not None:                     # chosen before (by this or an earlier process): no timing
             self._select(name, rec['index'])
             self.build_times[name] = [float('inf') if t is None else t for t in rec.get('ms', [])] or None
+            self.build_source[name] = 'stored choice'
             return
         saved = [a.clone() for a in accumulators]
         times = [float('inf')] * n
         usable = [True] * n
         # rounds over all candidates (the first untimed) rather than one candidate after the other: the
         # clock ramps up over the first launches, and whoever ran first would be timed on a cold chip
-        for rnd in range(4):
+        for rnd in range(self._tune_rounds):
             for i in range(n):
                 if not usable[i]:
                     continue
                 self._select(name, i)
                 try:
-                    e0, e1 = th.cuda.Event(enable_timing=True), th.cuda.Event(enable_timing=True)
-                    e0.record()
-                    self._launch(name, tensors)
-                    e1.record()
-                    e1.synchronize()
+                    ms = self._timed_launch(name, tensors)
                     if rnd:
-                        times[i] = min(times[i], e0.elapsed_time(e1))
+                        times[i] = min(times[i], ms)
                 except runtime.RuntimeError_:
                     if i == 0:
                         raise                   # the first-ranked build must be launchable
@@ -574,6 +687,7 @@ class CompiledPlan:
         best = min(range(len(times)), key=times.__getitem__)
         self._select(name, best)
         self.build_times[name] = times
+        self.build_source[name] = 'timed in this process'
         PICKS.put(pkey, best, times)
         for a, s_ in zip(accumulators, saved):
             a.copy_(s_)

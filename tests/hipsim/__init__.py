@@ -1,33 +1,49 @@
 """CPU execution of the emitted HIP kernels (test tool).
 
-`SimPlan` is `flex_rnn_amd.launch.CompiledPlan` with the two device-facing steps swapped:
+`SimPlan` is `flex_rnn_amd.launch.CompiledPlan` with the device-facing steps swapped:
 kernels are compiled for the host against `hipsim.h` (fibers as GPU threads, see there) and a
 launch runs the workgroups one after another on CPU tensors.  Every tensor of a launch is
-copied into a buffer that ends (or, on a second pass, starts) at an inaccessible guard page, so
+copied into a buffer that ends (or, on a second pass, starts) at an inaccessible guard region, so
 an out-of-bounds access by the kernel kills the process with SIGSEGV; callers run it in a
-subprocess.  All host logic (allocation, argument packing, launch order, scratch handling) is
-the product's own code.
+subprocess.  All host logic - allocation of results and hidden buffers, the choice among the
+candidate builds of a kernel with its re-registration of grid and argument layout (`_tune`,
+`_select`), argument packing, the launch audit, launch order, scratch handling - is the product's
+own code.
+
+Environment: HIPSIM_SEED=<n> shuffles threads and workgroups (hipsim.h); HIPSIM_BOUNDS=1 checks
+every index into a declared array; HIPSIM_UNINIT=1 builds with clang and fills every uninitialised
+local variable with a NaN pattern; HIPSIM_CANDIDATES=1 makes `SimPlan` hold every candidate build
+the product would time on a GPU and run each of them once per kernel before settling on one.
 """
 from __future__ import annotations
 
 import ctypes
 import hashlib
 import os
-import struct
+import re
 import subprocess
 import tempfile
 
 import torch as th
 
-from flex_rnn_amd.launch import CompiledPlan, kernel_specs, _strides5
+from flex_rnn_amd import launch
+from flex_rnn_amd.launch import CompiledPlan, kernel_specs
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _CACHE = os.path.join(tempfile.gettempdir(), 'frnn_hipsim')
+_CLANG = '/opt/rocm/lib/llvm/bin/clang++'
+LDS_LIMIT = 160 * 1024          # bytes of LDS a gfx950 workgroup may use
+
+_SHARED_DECL = re.compile(r'__shared__\s+float\s+(\w+)((?:\[[^\]]+\])+);')
 
 
 def _compile_host(spec) -> str:
     src = spec.source.replace('#include <hip/hip_runtime.h>', '#include "hipsim.h"')
     assert 'hipsim.h' in src
+    src = re.sub(r'__attribute__\(\(amdgpu_waves_per_eu\([^)]*\)\)\)', '', src)      # (an occupancy request; means nothing on the host)
+    # LDS arrays start a workgroup with undefined contents: poison each one where it is declared
+    src, n = _SHARED_DECL.subn(lambda m: f'__shared__ float {m.group(1)}{m.group(2)}; sim_lds_poison({m.group(1)}, sizeof({m.group(1)}));', src)
+    assert n == src.count('__shared__'), 'a __shared__ declaration the harness does not recognise'
     src += f'''
 extern "C" int sim_launch_{spec.name}(const void* argbuf, int gx, int gy, int gz, int bx) {{
   Args A;
@@ -39,7 +55,12 @@ extern "C" int sim_args_size_{spec.name}() {{ return (int)sizeof(Args); }}
     hdr = open(os.path.join(_HERE, 'hipsim.h')).read()
     # HIPSIM_BOUNDS=1: every index into a declared array (registers, LDS) is checked, a bad one traps
     extra = ['-fsanitize=bounds', '-fsanitize-undefined-trap-on-error'] if os.environ.get('HIPSIM_BOUNDS', '0') == '1' else []
-    key = hashlib.sha256((hdr + src + ' '.join(extra)).encode()).hexdigest()[:20]
+    cxx = 'g++'
+    if os.environ.get('HIPSIM_UNINIT', '0') == '1':
+        # registers hold no zeros either: every local variable the code does not initialise starts as a NaN pattern
+        assert os.access(_CLANG, os.X_OK), f'HIPSIM_UNINIT needs {_CLANG}'
+        cxx, extra = _CLANG, extra + ['-ftrivial-auto-var-init=pattern']
+    key = hashlib.sha256((hdr + src + cxx + ' '.join(extra)).encode()).hexdigest()[:20]
     os.makedirs(_CACHE, exist_ok=True)
     so = os.path.join(_CACHE, f'{spec.name}_{key}.so')
     if not os.path.isfile(so):
@@ -47,45 +68,93 @@ extern "C" int sim_args_size_{spec.name}() {{ return (int)sizeof(Args); }}
         with open(cpp, 'w') as f:
             f.write(src)
         tmp = so + f'.tmp{os.getpid()}'
-        cmd = ['g++', '-O1', '-std=c++17', '-shared', '-fPIC', '-w', *extra, '-I', _HERE, cpp, '-o', tmp]
+        cmd = [cxx, '-O1', '-std=c++17', '-shared', '-fPIC', '-w', *extra, '-I', _HERE, cpp, '-o', tmp]
         subprocess.run(cmd, check=True)
         os.replace(tmp, so)
     return so
 
 
+class SimKernel:
+    """A host build of one emitted kernel; stands where the product holds a `runtime.Kernel`."""
+
+    def __init__(self, spec):
+        self.spec = spec
+        self.lib = ctypes.CDLL(_compile_host(spec))
+        self.lib.sim_alloc.restype = ctypes.c_void_p
+        self.lib.sim_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]
+        self.lib.sim_free.argtypes = [ctypes.c_void_p]
+        self.lib.sim_lds_peak_bytes.restype = ctypes.c_size_t
+        self.fn = getattr(self.lib, f'sim_launch_{spec.name}')
+        self.fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        self.arg_bytes = int(getattr(self.lib, f'sim_args_size_{spec.name}')())
+
+
 class SimPlan(CompiledPlan):
+    _on_gpu = False
+    _tune_rounds = 2
+
     def __init__(self, plan, state_meta=None, against_end=True):
         self.plan = plan
         self.state_meta = state_meta
         self.against_end = against_end
-        self.kernels = {}
-        # HIPSIM_PREFETCH selects the gradient kernel's variant with that many checkpoint rows in flight
-        specs = kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4')))
-        from flex_rnn_amd.emit_hip import Emitter
-        specs.append(Emitter(plan).fw(save=False))          # the inference kernel, used by forward_only()
+        self.device = None
+        self.profile_events = None
+        self.kernels, self.modules = {}, []
+        self.builds, self.build_times, self._grid, self._packer = {}, {}, {}, {}
+        self.build_source = {}
+        self.launches = []          # (kernel name, candidate number) of every launch, in order
+        self._fixed = {}
+        self._tune_on = True
+        self.lds_peak = {}
+        if plan.B == 0 or plan.T == 0:
+            return
+        candidates = os.environ.get('HIPSIM_CANDIDATES', '0') == '1'
+        if candidates:
+            # every candidate build the product would time on the first call of a problem large enough to time the
+            # code-generation knobs too
+            old, launch.TUNE_KNOBS_FROM = launch.TUNE_KNOBS_FROM, 0
+            try:
+                sets = {'frnn_fw': launch.row_kernel_specs(plan, False), 'frnn_bw1': launch.row_kernel_specs(plan, True),
+                        'frnn_fwi': launch.row_kernel_specs(plan, False, save=False)}
+            finally:
+                launch.TUNE_KNOBS_FROM = old
+            if launch.needs_gradient_kernel(plan.part):
+                sets['frnn_bw2'] = launch.gradient_kernel_specs(plan)
+        else:
+            # HIPSIM_PREFETCH selects the gradient kernel's variant with that many checkpoint rows in flight
+            specs = kernel_specs(plan, prefetch=int(os.environ.get('HIPSIM_PREFETCH', '4')))
+            from flex_rnn_amd.emit_hip import Emitter
+            specs.append(Emitter(plan).fw(save=False))          # the inference kernel, used by forward_only()
+            sets = {s_.name: [s_] for s_ in specs}
         from concurrent.futures import ThreadPoolExecutor
-        with ThreadPoolExecutor(max_workers=len(specs)) as pool:      # host compiler runs side by side
-            list(pool.map(_compile_host, specs))
-        for spec in specs:
-            self._add_kernel(spec)
+        flat = [s_ for v in sets.values() for s_ in v]
+        with ThreadPoolExecutor(max_workers=min(8, len(flat))) as pool:      # host compiler runs side by side
+            list(pool.map(_compile_host, flat))
+        for name, specs in sets.items():
+            self.builds[name] = [(s_, SimKernel(s_), None) for s_ in specs]
+            if len(specs) > 1:
+                self._tune_pending = set(self._tune_pending) | {name}
+            self._select(name, 0)
 
-    def _tune(self, name, tensors, accumulators=()):
-        pass
+    def _device_name(self):
+        return 'hipsim'
 
-    def _add_kernel(self, spec):
-        lib = ctypes.CDLL(_compile_host(spec))
-        lib.sim_alloc.restype = ctypes.c_void_p
-        lib.sim_alloc.argtypes = [ctypes.c_size_t, ctypes.c_int]
-        lib.sim_free.argtypes = [ctypes.c_void_p]
-        fn = getattr(lib, f'sim_launch_{spec.name}')
-        fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]
-        self.kernels[spec.name] = (spec, lib, fn)
+    def _capturing(self):
+        return False
+
+    def _timed_launch(self, kname, tensors):
+        """A launch of the selected candidate; the "time" makes the last candidate the winner of `_tune`, so
+        that the launch after the timing rounds runs a build other than the first."""
+        self._launch(kname, tensors)
+        spec = self.kernels[kname][0]
+        index = next(i for i, b in enumerate(self.builds[kname]) if b[0] is spec)
+        return float(len(self.builds[kname]) - index)
 
     def _launch(self, kname, tensors):
-        spec, lib, fn = self.kernels[kname]
-        pl = self.plan
-        buf = bytearray()
-        staged = []
+        spec, kern = self.kernels[kname]
+        self.launches.append((kname, next(i for i, b in enumerate(self.builds[kname]) if b[0] is spec)))
+        lib = kern.lib
+        staged, guarded = [], {}
         for name in spec.tensors:
             t = tensors[name]
             assert not t.is_cuda
@@ -95,22 +164,22 @@ class SimPlan(CompiledPlan):
             p = lib.sim_alloc(nbytes, 1 if self.against_end else 0)
             assert p, 'sim_alloc failed'
             if nbytes:
-                flat = th.as_strided(t, (span,), (1,))
-                ctypes.memmove(p, flat.data_ptr(), nbytes)
+                ctypes.memmove(p, th.as_strided(t, (span,), (1,)).data_ptr(), nbytes)
+                raw = th.frombuffer((ctypes.c_char * nbytes).from_address(p), dtype=t.dtype, count=span)
+                guarded[name] = th.as_strided(raw, t.shape, t.stride())
+            else:
+                guarded[name] = t
             staged.append((t, p, nbytes, span))
-            buf += struct.pack('<q5q', p, *_strides5(t))
-        if not spec.tensors:
-            buf += struct.pack('<q5q', 0, 0, 0, 0, 0, 0)
-        buf += struct.pack('<5q', pl.B, pl.T, pl.H, pl.M, pl.nchunks)
-        size = getattr(lib, f'sim_args_size_{spec.name}')()
-        assert len(buf) == size, (size, len(buf))      # the block must match the kernel's parameter list
-        env = dict(B=pl.B, T=pl.T, H=pl.H, M=pl.M, nch=pl.nchunks)
-        grid = tuple(int(eval(g, {}, env)) for g in spec.grid)
+        buf, _ = self._pack(kname, guarded)         # (the product's packing and, with FLEX_RNN_CHECK=1, its audit)
+        assert len(buf) == kern.arg_bytes, (kern.arg_bytes, len(buf))      # the block must match the kernel's parameter list
+        grid = self._grid[kname]
         cbuf = ctypes.create_string_buffer(bytes(buf), len(buf))
-        rc = fn(cbuf, grid[0], grid[1], grid[2], spec.block)
+        rc = kern.fn(cbuf, grid[0], grid[1], grid[2], spec.block)
         assert rc == 0, f'hipsim launch of {kname} failed'
+        peak = int(lib.sim_lds_peak_bytes())
+        self.lds_peak[kname] = max(self.lds_peak.get(kname, 0), peak)
+        assert peak <= LDS_LIMIT, f'{kname} uses {peak} bytes of LDS per workgroup, gfx950 has {LDS_LIMIT}'
         for t, p, nbytes, span in staged:
             if nbytes:
-                flat = th.as_strided(t, (span,), (1,))
-                ctypes.memmove(flat.data_ptr(), p, nbytes)
+                ctypes.memmove(th.as_strided(t, (span,), (1,)).data_ptr(), p, nbytes)
             lib.sim_free(p)

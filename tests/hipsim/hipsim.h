@@ -1,13 +1,20 @@
 // hipsim: run an emitted HIP kernel on the CPU, one workgroup at a time.  TEST TOOL ONLY.
 //
 // Every GPU thread of a workgroup is a ucontext fiber on one OS thread.  A barrier yields to
-// the scheduler, which resumes the fibers round-robin, so "resume every fiber once" is one
-// barrier phase.  Cross-lane operations (DPP, shuffles) are an exchange through a per-block
-// array bracketed by two such barriers, which is valid because the kernels only reduce in
-// workgroup-uniform control flow.  `__shared__` becomes `static` (workgroups run one after
-// another).  Buffers handed to the kernel come from sim_alloc(), which places them against a
-// PROT_NONE guard page, so an out-of-bounds access ends the process with SIGSEGV instead of
-// passing silently.
+// the scheduler, which resumes every fiber once per barrier phase: in index order, or - with
+// HIPSIM_SEED set to a non-zero number - in a fresh random order in every phase, with the
+// workgroups of the grid shuffled as well, so that code which only works for one order of the
+// threads between two barriers (a missing barrier, a read of LDS before its write) or of the
+// workgroups gives wrong results for some seed.  Cross-lane operations (DPP, shuffles) are an
+// exchange through a per-block array bracketed by two such barriers, which is valid because the
+// kernels only reduce in workgroup-uniform control flow.  `__shared__` becomes `static`
+// (workgroups run one after another); the harness's build step adds a call of sim_lds_poison()
+// after every such declaration, which fills the array with NaNs when a workgroup first reaches
+// it: LDS holds no zeros at the start of a workgroup and keeps nothing from the one before.
+// Buffers handed to the kernel come from sim_alloc(), which places them between two
+// inaccessible regions of SIM_GUARD bytes each, so an access outside a tensor - by less than that -
+// ends the process with SIGSEGV (the handler names the address, the nearest tensor, block and thread)
+// instead of passing silently.
 #pragma once
 #include <math.h>
 #include <stdint.h>
@@ -18,8 +25,12 @@
 #include <ucontext.h>
 #include <unistd.h>
 
+#include <signal.h>
+
 #include <algorithm>
 #include <functional>
+#include <map>
+#include <random>
 #include <vector>
 
 struct sim_dim3 { unsigned x, y, z; };
@@ -56,45 +67,72 @@ static inline void sim_barrier() {
 }
 #define __syncthreads() sim_barrier()
 
+static unsigned long sim_block_epoch = 0;      // counts workgroups; LDS arrays are poisoned once per workgroup
+static size_t sim_lds_bytes = 0, sim_lds_peak = 0;
+
+// Called right after the declaration of a `__shared__` array: the first thread of a workgroup that gets
+// there fills it with NaNs (what a workgroup finds in LDS is undefined) and counts its size.
+static inline void sim_lds_poison(void* p, size_t nbytes) {
+  static std::map<void*, unsigned long> seen;
+  unsigned long& e = seen[p];
+  if (e == sim_block_epoch) return;
+  e = sim_block_epoch;
+  uint32_t* w = (uint32_t*)p;
+  for (size_t i = 0; i < nbytes / 4; i++) w[i] = 0x7fc0dead;
+  sim_lds_bytes += nbytes;
+  sim_lds_peak = std::max(sim_lds_peak, sim_lds_bytes);
+}
+extern "C" size_t sim_lds_peak_bytes() { return sim_lds_peak; }
+
 static int sim_run_grid(const std::function<void()>& body, int gx, int gy, int gz, int bx) {
   const size_t STACK = 256 * 1024;
+  const char* seed_env = getenv("HIPSIM_SEED");
+  const unsigned long seed = seed_env ? strtoul(seed_env, nullptr, 10) : 0;
+  std::mt19937 rng((unsigned)seed);
   std::vector<char*> stacks(bx);
   for (int i = 0; i < bx; i++) stacks[i] = (char*)malloc(STACK);
   sim_body = body;
   blockDim = {(unsigned)bx, 1, 1};
   gridDim = {(unsigned)gx, (unsigned)gy, (unsigned)gz};
-  for (int bz = 0; bz < gz; bz++)
-    for (int by = 0; by < gy; by++)
-      for (int bxi = 0; bxi < gx; bxi++) {
-        blockIdx = {(unsigned)bxi, (unsigned)by, (unsigned)bz};
-        sim_fibers.assign(bx, ucontext_t());
-        sim_done.assign(bx, 0);
-        for (int i = 0; i < bx; i++) {
-          getcontext(&sim_fibers[i]);
-          sim_fibers[i].uc_stack.ss_sp = stacks[i];
-          sim_fibers[i].uc_stack.ss_size = STACK;
-          sim_fibers[i].uc_link = &sim_sched_ctx;
-          makecontext(&sim_fibers[i], sim_trampoline, 0);
-        }
-        int remaining = bx;
-        while (remaining > 0) {
-          int finished_now = 0, alive = 0;
-          for (int i = 0; i < bx; i++) {
-            if (sim_done[i]) continue;
-            alive++;
-            sim_cur = i;
-            threadIdx = {(unsigned)i, 0, 0};
-            swapcontext(&sim_sched_ctx, &sim_fibers[i]);
-            if (sim_done[i]) finished_now++;
-          }
-          // all threads of a workgroup must leave together (no early exit before a barrier)
-          if (finished_now != 0 && finished_now != alive) {
-            fprintf(stderr, "hipsim: threads of one workgroup ended at different barriers\n");
-            return 1;
-          }
-          remaining -= finished_now;
-        }
+  std::vector<long> blocks((size_t)gx * gy * gz);
+  for (size_t i = 0; i < blocks.size(); i++) blocks[i] = (long)i;
+  if (seed) std::shuffle(blocks.begin(), blocks.end(), rng);
+  std::vector<int> order(bx);
+  for (long blk : blocks) {
+    blockIdx = {(unsigned)(blk % gx), (unsigned)((blk / gx) % gy), (unsigned)(blk / ((long)gx * gy))};
+    sim_block_epoch++;
+    sim_lds_bytes = 0;
+    sim_fibers.assign(bx, ucontext_t());
+    sim_done.assign(bx, 0);
+    for (int i = 0; i < bx; i++) {
+      getcontext(&sim_fibers[i]);
+      sim_fibers[i].uc_stack.ss_sp = stacks[i];
+      sim_fibers[i].uc_stack.ss_size = STACK;
+      sim_fibers[i].uc_link = &sim_sched_ctx;
+      makecontext(&sim_fibers[i], sim_trampoline, 0);
+    }
+    int remaining = bx;
+    while (remaining > 0) {
+      int finished_now = 0, alive = 0;
+      for (int i = 0; i < bx; i++) order[i] = i;
+      if (seed) std::shuffle(order.begin(), order.end(), rng);
+      for (int k = 0; k < bx; k++) {
+        const int i = order[k];
+        if (sim_done[i]) continue;
+        alive++;
+        sim_cur = i;
+        threadIdx = {(unsigned)i, 0, 0};
+        swapcontext(&sim_sched_ctx, &sim_fibers[i]);
+        if (sim_done[i]) finished_now++;
       }
+      // all threads of a workgroup must leave together (no early exit before a barrier)
+      if (finished_now != 0 && finished_now != alive) {
+        fprintf(stderr, "hipsim: threads of one workgroup ended at different barriers\n");
+        return 1;
+      }
+      remaining -= finished_now;
+    }
+  }
   for (int i = 0; i < bx; i++) free(stacks[i]);
   return 0;
 }
@@ -155,11 +193,13 @@ static inline float __shfl_xor(float v, int mask, int width = 64) {
   return f;
 }
 
-template <class T> static inline T __hip_atomic_fetch_add(T* p, T v, int, int) {
+// (a macro, not a function of that name: clang knows the name as a builtin)
+template <class T> static inline T sim_atomic_fetch_add(T* p, T v, int, int) {
   T o = *p;
   *p = o + v;
   return o;
 }
+#define __hip_atomic_fetch_add sim_atomic_fetch_add
 
 // ------------------------------------------------------------------ math + narrow floats
 #define __expf(x) expf(x)
@@ -223,23 +263,50 @@ struct sim_half {
 #define _Float16 sim_half
 
 // ------------------------------------------------------------------ guarded allocation
-#include <map>
 static std::map<void*, std::pair<void*, size_t>> sim_maps;
 
-// `nbytes` of read/write memory with an inaccessible page on both sides.  With `against_end`
-// the block ends (up to 16-byte alignment) at the trailing guard page, otherwise it starts
-// right after the leading one.
+// `nbytes` of read/write memory with SIM_GUARD inaccessible bytes on both sides (address space only).  With
+// `against_end` the block ends (up to 16-byte alignment) at the trailing guard, otherwise it starts right
+// after the leading one.
+static const size_t SIM_GUARD = (size_t)1 << 30;
+struct sim_block_info { char* lo; size_t nbytes; };
+static std::vector<sim_block_info> sim_live;
+
+static void sim_segv(int, siginfo_t* si, void*) {
+  char* a = (char*)si->si_addr;
+  fprintf(stderr, "hipsim: access outside every tensor at %p, block (%u,%u,%u) thread %u\n", (void*)a, blockIdx.x, blockIdx.y,
+          blockIdx.z, threadIdx.x);
+  for (size_t i = 0; i < sim_live.size(); i++) {
+    long before = (long)(sim_live[i].lo - a), after = (long)(a - (sim_live[i].lo + sim_live[i].nbytes));
+    if (before > 0 && before <= (long)SIM_GUARD) fprintf(stderr, "  %ld bytes before tensor #%zu (%zu bytes)\n", before, i, sim_live[i].nbytes);
+    if (after >= 0 && after < (long)SIM_GUARD) fprintf(stderr, "  %ld bytes past the end of tensor #%zu (%zu bytes)\n", after, i, sim_live[i].nbytes);
+  }
+  _exit(139);
+}
+
 extern "C" void* sim_alloc(size_t nbytes, int against_end) {
+  static bool handler = false;
+  if (!handler) {
+    handler = true;
+    static char altstack[64 * 1024];
+    stack_t ss = {altstack, 0, sizeof(altstack)};
+    sigaltstack(&ss, nullptr);
+    struct sigaction sa;
+    memset(&sa, 0, sizeof(sa));
+    sa.sa_sigaction = sim_segv;
+    sa.sa_flags = SA_SIGINFO | SA_ONSTACK;
+    sigaction(SIGSEGV, &sa, nullptr);
+  }
   size_t page = (size_t)sysconf(_SC_PAGESIZE);
   size_t body = (nbytes + page - 1) / page * page;
   if (body == 0) body = page;
-  char* base = (char*)mmap(nullptr, body + 2 * page, PROT_READ | PROT_WRITE, MAP_PRIVATE | MAP_ANONYMOUS, -1, 0);
+  char* base = (char*)mmap(nullptr, body + 2 * SIM_GUARD, PROT_NONE, MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0);
   if (base == MAP_FAILED) return nullptr;
-  mprotect(base, page, PROT_NONE);
-  mprotect(base + page + body, page, PROT_NONE);
-  char* p = base + page;
+  mprotect(base + SIM_GUARD, body, PROT_READ | PROT_WRITE);
+  char* p = base + SIM_GUARD;
   if (against_end) p += (body - nbytes) & ~(size_t)15;
-  sim_maps[p] = {base, body + 2 * page};
+  sim_maps[p] = {base, body + 2 * SIM_GUARD};
+  sim_live.push_back({p, nbytes});
   return p;
 }
 
@@ -248,4 +315,6 @@ extern "C" void sim_free(void* p) {
   if (it == sim_maps.end()) return;
   munmap(it->second.first, it->second.second);
   sim_maps.erase(it);
+  for (size_t i = 0; i < sim_live.size(); i++)
+    if (sim_live[i].lo == (char*)p) { sim_live.erase(sim_live.begin() + i); break; }
 }

@@ -11,6 +11,13 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, os.path.dirname(HERE))
 sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
+if os.environ.get('HIPSIM_CANDIDATES', '0') == '1':
+    # every candidate is run; the choice among them goes to a scratch directory, never to the product's cache
+    import tempfile
+    os.environ['FLEX_RNN_CACHE'] = tempfile.mkdtemp(prefix='frnn_hipsim_picks_')
+    os.environ['FLEX_RNN_RETUNE'] = '1'
+os.environ.setdefault('FLEX_RNN_CHECK', '1')        # the product's launch audit runs on every simulated launch
+
 import torch as th
 
 import cases
@@ -62,7 +69,8 @@ def main():
     want = list(want[0]) + list(want[1]) + list(want[2]) + list(want[3])
     print(f'{name} {dims} {dt} tile={plan.tile}', flush=True)
     worst = max(recurrence.assert_all_close(got, want, tol, name))
-    print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e}')
+    ran = sorted({f'{k}#{i}' for k, i in sp.launches})
+    print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e} lds={sp.lds_peak} builds run: {" ".join(ran)}')
 
 
 if __name__ == '__main__':
