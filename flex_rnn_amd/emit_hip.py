@@ -375,6 +375,163 @@ class _Stager:
         return out
 
 
+class _Prologue:
+    """Values of a step that do not vary along the state's rows and are not plain inputs - a gate's sigmoid, a
+    softplus step size, an L2-normalised key, anything a traced layer moved into the step - evaluated by the
+    workgroup once per (timestep, column) right after a block of timesteps was staged, instead of by every row group
+    of every wave inside the step.  `front` are the outermost such values (those a value with a row extent, or a
+    result, reads); the step takes them from LDS like staged operands.
+
+    On the way to them the graph is cut at every value that is one number per timestep: sums over the columns (the
+    squared norm of a key) and the outermost values computed from scalars alone (a gate).  Cuts are grouped into
+    levels by what they depend on; a level's sums are formed by groups of 16 lanes, one timestep per group, its
+    scalar values by one lane per timestep, then a barrier.  A last pass evaluates the front values per
+    (timestep, column) from the raw LDS rows and the cuts.  Inputs without a time axis are put into LDS once, before
+    the time loop."""
+
+    def __init__(self, em: 'Emitter', front, tag: str, TS: int, NT: int, A: '_Args'):
+        p, joint = em.p, em.p.joint
+        self.em, self.front, self.tag, self.TS, self.NT, self.A = em, list(front), tag, TS, NT, A
+        self.jext = em.jext
+        nm = joint.node_map()
+        need, stack = set(), list(front)
+        while stack:
+            v = stack.pop()
+            if v in need:
+                continue
+            need.add(v)
+            if v in nm:
+                stack.extend(nm[v].value_args())
+        nodes = [n for n in joint.nodes if n.name in need]
+        self.inputs = [i for i in range(p.ninputs) if p.in_names[i] in need]
+        for i in self.inputs:
+            assert not em.in_ext(i)[0], p.in_names[i]
+        # cuts: sums, and scalar values that a per-column value (or the step) reads
+        cuts = []
+        for n in nodes:
+            if n.op == 'sum':
+                cuts.append(n.name)
+            elif n.ext == (False, False) and n.op != 'const' and (
+                    n.name in front or any(n.name in m.value_args() and m.ext[1] for m in nodes)):
+                cuts.append(n.name)
+        # level of a cut: one more than the highest level among the cuts it is computed from
+        dep, level = {}, {}
+        for n in nodes:
+            d = set()
+            for a in n.value_args():
+                d |= ({a} if a in cuts else set()) | dep.get(a, set())
+            dep[n.name] = d
+        for c in cuts:
+            level[c] = 1 + max((level[d] for d in dep[c]), default=-1)
+        self.cuts = cuts
+        self.fns, self.levels = [], []          # device functions; per level: (sum pass or None, scalar pass or None)
+        for lv in range(1 + max(level.values(), default=-1)):
+            done = [c for c in cuts if level[c] < lv]
+            passes = []
+            for kind in ('sum', 'scalar'):
+                mine = [c for c in cuts if level[c] == lv and (nm[c].op == 'sum') == (kind == 'sum')]
+                if not mine:
+                    passes.append(None)
+                    continue
+                outs = [nm[c].args[0] for c in mine] if kind == 'sum' else mine
+                fname = f'{tag}_p{kind}{lv}'
+                g = joint.extract(fname, outs, cut=done)
+                src, used = emit_graph_fn(g, fname, 1, 1, [(False, kind == 'sum')] * len(outs), 'grp_allreduce<1>', em.invariant)
+                self.fns.append(src)
+                passes.append((fname, used, mine))
+            self.levels.append(passes)
+        g = joint.extract(f'{tag}_pfront', self.front, cut=cuts)
+        src, used = emit_graph_fn(g, f'{tag}_pfront', 1, 1, [self.jext[f] for f in self.front], 'grp_allreduce<1>', em.invariant)
+        self.fns.append(src)
+        self.final = (f'{tag}_pfront', used)
+
+    def source(self) -> str:
+        return '\n'.join(self.fns)
+
+    def decls(self) -> str:
+        em = self.em
+        out = ''
+        for j in range(len(self.cuts)):
+            out += f'  __shared__ float s_pc{j}[{self.TS}];\n'
+        for q, f in enumerate(self.front):
+            out += f'  __shared__ float s_d{q}[{self.TS}][{em.NP if self.jext[f][1] else 1}];\n'
+        for i in self.inputs:
+            if not em.tdep[i]:
+                out += f'  __shared__ float s_k{i}[{em.NP if em.in_ext(i)[1] else 1}];\n'
+        return out
+
+    def init(self) -> str:
+        """Inputs without a time axis into LDS, and the padding columns of the front arrays cleared (once; a barrier
+        follows before anything reads them)."""
+        em, A = self.em, self.A
+        out = ''
+        for i in self.inputs:
+            if em.tdep[i]:
+                continue
+            dt = DT_CODE[em.plan.in_dtypes[i]]
+            if em.in_ext(i)[1]:
+                out += (f'  for (int x_ = tid; x_ < {em.N}; x_ += {self.NT}) s_k{i}[x_] = '
+                        f'ldf<{dt}>({A.p(f"in{i}")}, {em._in_index(A, i, t="0", n="x_")});\n')
+            else:
+                out += f'  if (tid == 0) s_k{i}[0] = ldf<{dt}>({A.p(f"in{i}")}, {em._in_index(A, i, t="0")});\n'
+        if em.pad:
+            pad = em.NP - em.N
+            for q, f in enumerate(self.front):
+                if self.jext[f][1]:
+                    out += (f'  for (int e_ = tid; e_ < {self.TS * pad}; e_ += {self.NT}) '
+                            f's_d{q}[e_ / {pad}][{em.N} + e_ % {pad}] = 0.0f;\n')
+        return out
+
+    def _value(self, v: str) -> str:
+        """Expression for graph value `v` at (timestep tt_, column x_)."""
+        em, p = self.em, self.em.p
+        if v in self.cuts:
+            return f's_pc{self.cuts.index(v)}[tt_]'
+        i = p.in_names.index(v)
+        col = 'x_' if em.in_ext(i)[1] else '0'
+        return f's_in{i}[tt_][{col}]' if em.tdep[i] else f's_k{i}[{col}]'
+
+    def _call(self, fname, used, outs) -> str:
+        args = ' '.join(f'float a{k}_[1][1]; a{k}_[0][0] = {self._value(v)};' for k, v in enumerate(used))
+        decl = ' '.join(f'float {o}[1][1];' for o in outs)
+        return f'{args} {decl} {fname}(' + ', '.join([f'a{k}_' for k in range(len(used))] + list(outs)) + ');'
+
+    def run(self, ind: str) -> str:
+        """The passes of one staged block; ends with a barrier."""
+        em, TS, NT = self.em, self.TS, self.NT
+        out = ''
+        for sums, scalars in self.levels:
+            if sums:
+                fname, used, mine = sums
+                outs = [f'o{k}_' for k in range(len(mine))]
+                out += (f'{ind}for (int tt_ = tid / 16; tt_ < {TS}; tt_ += {NT // 16}) {{ '
+                        + ' '.join(f'float s{k}_ = 0.0f;' for k in range(len(mine))) + '\n'
+                        f'{ind}  for (int x_ = tid % 16; x_ < {em.N}; x_ += 16) {{ {self._call(fname, used, outs)} '
+                        + ' '.join(f's{k}_ += o{k}_[0][0];' for k in range(len(mine))) + ' }\n'
+                        + ''.join(f'{ind}  s{k}_ = grp_allreduce<16>(s{k}_);\n' for k in range(len(mine)))
+                        + f'{ind}  if ((tid & 15) == 0) {{ ' + ' '.join(f's_pc{self.cuts.index(c)}[tt_] = s{k}_;' for k, c in enumerate(mine))
+                        + ' } }\n')
+            if scalars:
+                fname, used, mine = scalars
+                outs = [f'o{k}_' for k in range(len(mine))]
+                out += (f'{ind}for (int tt_ = tid; tt_ < {TS}; tt_ += {NT}) {{ const int x_ = 0; (void)x_; {self._call(fname, used, outs)} '
+                        + ' '.join(f's_pc{self.cuts.index(c)}[tt_] = o{k}_[0][0];' for k, c in enumerate(mine)) + ' }\n')
+            out += f'{ind}__syncthreads();\n'
+        fname, used = self.final
+        outs = [f'o{q}_' for q in range(len(self.front))]
+        vec = [(q, f) for q, f in enumerate(self.front) if self.jext[f][1]]
+        sca = [(q, f) for q, f in enumerate(self.front) if not self.jext[f][1]]
+        stores = ' '.join(f's_d{q}[tt_][x_] = o{q}_[0][0];' for q, f in vec)
+        if sca:
+            stores += ' if (x_ == 0) { ' + ' '.join(f's_d{q}[tt_][0] = o{q}_[0][0];' for q, f in sca) + ' }'
+        total = TS * em.N if vec else TS
+        step = em.N if vec else 1
+        out += (f'{ind}for (int e_ = tid; e_ < {total}; e_ += {NT}) {{ const int tt_ = e_ / {step}, x_ = e_ % {step}; (void)x_;\n'
+                f'{ind}  {self._call(fname, used, outs)} {stores} }}\n'
+                f'{ind}__syncthreads();\n')
+        return out
+
+
 def _col_expr(C: int, L: int) -> str:
     """Column owned by (lane-in-group l, element c).  With C >= 4 a lane owns float4
     pieces, interleaved across the group so that 16 lanes x 16 B is one contiguous row
@@ -448,6 +605,19 @@ class Emitter:
             for n in g.nodes:
                 if n.name in pure and n.name not in front and (
                         n.name in g.outputs or any(n.name in m.value_args() and m.name not in pure for m in g.nodes)):
+                    front.append(n.name)
+        return front
+
+    def _prologue_front(self, graphs):
+        """The outermost values of `graphs` that do not vary along the state's rows and are not plain inputs or
+        constants: those read by a value with a row extent, or returned.  What `_row_front` finds is the special case
+        that needs no pass of its own (values of one column of staged row inputs, no sums)."""
+        front = []
+        for g in graphs:
+            for n in g.nodes:
+                if n.ext[0] or n.op == 'const' or n.name in front:
+                    continue
+                if n.name in g.outputs or any(n.name in m.value_args() and m.ext[0] for m in g.nodes):
                     front.append(n.name)
         return front
 
@@ -598,6 +768,10 @@ class Emitter:
         st_ext = [self.jext[s] for s in p.st_names]
         out_exts = [(st_ext[0][0], False)] * nout + st_ext + [(st_ext[0][0], False)] * naux
         rfront = self._row_front([g])
+        pro = None
+        if sorted(rfront) != sorted(self._prologue_front([g])):        # sums or scalars on the way: a pass of its own
+            pro = _Prologue(self, self._prologue_front([g]), 'fw', TS, NT, A)
+            rfront = pro.front
         if rfront:
             g = g.extract('fw', g.outputs, cut=rfront)
         fn_src, used = emit_graph_fn(g, 'fw_step', R, C, out_exts, f'grp_allreduce<{L}>', self.invariant, self.colmask, self._lane_prolog())
@@ -607,12 +781,15 @@ class Emitter:
         # staging buffers
         tail = plan.T % TS != 0
         stg = _Stager(TS, NT, tail)
-        for i in used_in:
+        for i in sorted(set(used_in) | set(pro.inputs if pro else ())):
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
-        if rfront:
+        if pro:
+            fn_src = pro.source() + '\n' + fn_src
+            body.append(pro.decls())
+        elif rfront:
             fn_src = self._stage_row_front(stg, A, rfront, set(used), MT, 'fw_rowpre') + '\n' + fn_src
-        body.append(stg.decls() + stg.bases() + stg.zero_pads())
+        body.append(stg.decls() + stg.bases() + stg.zero_pads() + (pro.init() if pro else ''))
         # Results of a chunk (outputs, saved row sums) go to LDS per step and from there to memory.  With `df` they leave during
         # the next chunk, from the other half of a double buffer, and the checkpoint is stored after the staged operands were
         # written to LDS: a wave that waits for its prefetched loads also waits for every store it has issued, so stores
@@ -668,6 +845,8 @@ class Emitter:
         body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
+        if pro:
+            body.append(pro.run('    '))
         body.append(f'    if (t0 + {TS} < T) {{\n' + stg.load(f't0 + {TS}', '      ') + '    }\n')
         if ck_late:
             body += checkpoint()
@@ -687,7 +866,7 @@ class Emitter:
                 i = p.in_names.index(nm_)
                 operands[nm_] = (f'x{i}', f's_in{i}', self.in_ext(i))
             elif nm_ in rfront:
-                operands[nm_] = (f'd{rfront.index(nm_)}', f's_d{rfront.index(nm_)}', (False, True))
+                operands[nm_] = (f'd{rfront.index(nm_)}', f's_d{rfront.index(nm_)}', self.jext[nm_])
         order = self._operand_order(g, list(operands), skip=p.st_names)
         body.append(f'#pragma unroll {max(1, getattr(t, "UR", 2))}\n    for (int tt = 0; tt < nt; tt++) {{\n')
         for nm_ in order:
@@ -769,6 +948,11 @@ class Emitter:
         out_exts = st_ext + [colx] * len(p.col_idx) + [colx] * ndaux + [(True, True)] * len(mats)
         restep_g = p.restep
         rfront = self._row_front([g, restep_g] if needs_state else [g])
+        pro = None
+        pfront = self._prologue_front([g, restep_g] if needs_state else [g])
+        if sorted(rfront) != sorted(pfront):        # sums or scalars on the way: a pass of its own (as in the forward kernel)
+            pro = _Prologue(self, pfront, 'bw', TS, NT, A)
+            rfront = pro.front
         if rfront:
             g = g.extract('dstep', g.outputs, cut=rfront)
             restep_g = restep_g.extract('restep', restep_g.outputs, cut=rfront)
@@ -787,7 +971,7 @@ class Emitter:
         body = []
         tail = plan.T % TS != 0
         stg = _Stager(TS, NT, tail)
-        for i in used_in:
+        for i in sorted(set(used_in) | set(pro.inputs if pro else ())):
             if self.tdep[i]:
                 self._stage_input(stg, A, i, MT)
         for k in used_aux:
@@ -798,9 +982,12 @@ class Emitter:
             stg.add(f's_dy{k}', MT, DT_CODE[plan.out_dtypes[k]], A.p(nm),
                     lambda tt, x, nm=nm: (f'(i64)b * {A.s(nm, 0)} + (i64)({tt}) * {A.s(nm, 1)} + (i64)h * {A.s(nm, 2)} + '
                                            f'(i64)min(mt * {MT} + {x}, M - 1) * {A.s(nm, 3)}'), A.s(nm, 1))
-        if rfront:
+        if pro:
+            fns.insert(0, pro.source())
+            body.append(pro.decls())
+        elif rfront:
             fns.insert(0, self._stage_row_front(stg, A, rfront, used_all, MT, 'bw_rowpre'))
-        body.append(stg.decls() + stg.bases() + stg.zero_pads())
+        body.append(stg.decls() + stg.bases() + stg.zero_pads() + (pro.init() if pro else ''))
         tdep_col = [i for i in p.col_idx if self.tdep[i]]
         const_col = [i for i in p.col_idx if not self.tdep[i]]
         # (as in the forward kernel: with `df` a chunk's column gradients and saved sums leave LDS during the next chunk,
@@ -879,6 +1066,8 @@ class Emitter:
         body.append('    __syncthreads();\n')
         body.append(stg.write('    '))
         body.append('    __syncthreads();\n')
+        if pro:
+            body.append(pro.run('    '))
         for k in range(nst if needs_state else 0):
             rr, cc = _dims(st_ext[k], R, C)
             body.append(f'    float Sh{k}_0[{rr}][{cc}];\n#pragma unroll\n    for (int r = 0; r < {rr}; r++)\n'
@@ -937,7 +1126,7 @@ class Emitter:
                 elif nm_ in rfront:
                     q = rfront.index(nm_)
                     v = f'd{q}_{tt}' if needs_state else f'd{q}'
-                    loads[nm_] = (v, f's_d{q}', (False, True))
+                    loads[nm_] = (v, f's_d{q}', self.jext[nm_])
                     call.append(v)
                 else:
                     raise AssertionError(nm_)
@@ -1106,8 +1295,12 @@ class Emitter:
         pre_src, pre_used = '', []
         cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
         if front:
-            pre_g = p.joint.extract('colpre', front, cut=set(cuts))
+            # (a per-row scalar may read a value computed once per chunk - a sum over a row input, say; such values are
+            # inputs here and reach the staging loop, which picks the timestep at run time, through a small LDS table)
+            pre_g = p.joint.extract('colpre', front, cut=set(cuts) | set(rfront))
             pre_src, pre_used = emit_graph_fn(pre_g, 'bw_colpre', 1, 1, [(True, False)] * len(front), red, self.invariant)
+            assert all(self.jext[v] == (False, False) for v in pre_used if v in rfront), 'a per-row scalar cannot read a per-column value'
+        g_tables = [q for q, f in enumerate(rfront) if f in pre_used]
         rpre_used = []
         if rfront:
             rpre_g = p.joint.extract('rowpre', rfront, cut=set(cuts))
@@ -1216,6 +1409,8 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
         def raw_value(v, tt, mexpr):
             """Global-memory value of graph input `v` (an input, saved sum or output gradient without
             a column extent) at timestep offset `tt` of the chunk and row `mexpr`."""
+            if v in rfront:
+                return f's_g{rfront.index(v)}[inst][{tt}]'
             if v in p.in_names:
                 i = p.in_names.index(v)
                 ext = self.in_ext(i)
@@ -1273,6 +1468,11 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
                 for q, f in enumerate(rfront):
                     if IPB == 1 and self.jext[f] == (False, False) and n_uniform * DT <= 32:      # (more would spill scalar registers)
                         b.append(f'  g{q}_{tt}[0][0] = wave_uniform(g{q}_{tt}[0][0]);\n')
+            for q in g_tables:
+                b.append(f'  __shared__ float s_g{q}[{IPB}][{DT}];\n')
+                if HB > 1:
+                    b.append('  __syncthreads();\n')
+                b.append('  if (n == 0) { ' + ' '.join(f's_g{q}[inst][{tt}] = g{q}_{tt}[0][0];' for tt in range(DT)) + ' }\n')
         # ---- per-row operands of the chunk go through LDS: staged once per row block by the
         # instance's own lanes (coalesced along m), read back per row as broadcast vectors
         rowops = []          # (lds name, loader(tt, mexpr) -> expr, register prefix)

@@ -21,8 +21,14 @@ OPS = ['rwkv7', 'rwkv6', 'gla', 'retention', 'delta_rule', 'gated_delta_rule', '
        'hgrn', 'mamba', 's4d', 'gsa', 'mlstm']
 
 
-def build(op, B, T, D, C, device):
-    """Returns (inputs, layer) where layer(*inputs) calls jit-compiled steps through adapters."""
+RAW_OPS = ['rwkv7', 'gla', 'delta_rule', 'gated_delta_rule', 'mamba2', 'mamba', 'hgrn']
+
+
+def build(op, B, T, D, C, device, raw=False):
+    """Returns (inputs, layer, steps) where layer(*inputs) calls jit-compiled steps through adapters.  With `raw`
+    (ops in RAW_OPS) the layer takes the projections as a model produces them and prepares them itself - sigmoid
+    and softplus gates, L2-normalised keys, decay parameters - before it adapts shapes and calls the step: the
+    form `flex_rnn_amd.layer` is for."""
     H = D // C
     g = th.Generator().manual_seed(0)
 
@@ -34,6 +40,85 @@ def build(op, B, T, D, C, device):
     def jit(name, fn):
         steps[name] = flex_rnn_amd.jit(fn)
         return steps[name]
+
+    if raw:
+        assert op in RAW_OPS, f'no raw-projection form of {op}'
+        if op == 'rwkv7':
+            inputs = tuple(randn(B, T, H, C) for _ in range(6)) + (randn(B, H, C, C),)
+            st = jit('step', ops.rwkv7)
+
+            def layer(r, w, k, v, a, b, s):
+                w = -F.softplus(-w) - 0.5                       # log of a decay in (0, exp(-0.5))
+                a = F.normalize(a, dim=-1)
+                b = -a * th.sigmoid(b)
+                r, w, k, v, a, b = [i.unsqueeze(-2) for i in (r, w, k, v, a, b)]
+                y, s = st(r, w, k, v.mT, a, b, s.mT)
+                return y, s.mT
+        elif op == 'gla':
+            inputs = tuple(randn(B, T, H, C) for _ in range(4)) + (randn(B, H, C, C),)
+            st = jit('step', ops.gla)
+
+            def layer(q, k, v, g_, s):
+                g_ = -F.softplus(-g_) / 16                      # log-sigmoid gate with the usual normaliser
+                q = q * C ** -0.5
+                q, k, v, g_ = [i.unsqueeze(-2) for i in (q, k, v, g_)]
+                y, s = st(q, k, v.mT, g_, s.mT)
+                return y, s.mT
+        elif op in ('delta_rule', 'gated_delta_rule'):
+            q, k, v = [randn(B, T, H, C) for _ in range(3)]
+            beta = randn(B, T, H)
+            if op == 'delta_rule':
+                inputs = (q, k, v, beta, randn(B, H, C, C))
+                st = jit('step', ops.delta_rule)
+
+                def layer(q, k, v, beta, s):
+                    k = F.normalize(k, dim=-1)
+                    beta = th.sigmoid(beta)
+                    q, k, v, beta = [i.unsqueeze(-2) for i in (q, k, v, beta.unsqueeze(-1))]
+                    y, s = st(q, k, v.mT, beta, s.mT)
+                    return y, s.mT
+            else:
+                inputs = (q, k, v, randn(B, T, H), beta, randn(H), randn(H), randn(B, H, C, C))
+                st = jit('step', ops.gated_delta_rule)
+
+                def layer(q, k, v, a, beta, A_log, dt_bias, s):
+                    q, k = F.normalize(q, dim=-1), F.normalize(k, dim=-1)
+                    gate = -A_log.exp() * F.softplus(a + dt_bias)          # log of the gate
+                    beta = th.sigmoid(beta)
+                    q, k, v, gate, beta = [i.unsqueeze(-2) for i in (q, k, v, gate.unsqueeze(-1), beta.unsqueeze(-1))]
+                    y, s = st(q, k, v.mT, gate, beta, s.mT)
+                    return y, s.mT
+        elif op == 'mamba2':
+            inputs = (randn(B, T, H, C), randn(B, T, H), randn(H), randn(H), randn(B, T, 1, C), randn(B, T, 1, C), randn(B, H, C, C))
+            st = jit('step', ops.mamba2)
+
+            def layer(x, dt, dt_bias, A_log, b, c, s):
+                dt = F.softplus(dt + dt_bias)
+                A = -A_log.exp()
+                x, dt, A, b, c = [i.unsqueeze(-2) for i in (x, dt.unsqueeze(-1), A[None, None, :, None], b, c)]
+                return st(x.mT, dt, A, b, c, s)
+        elif op == 'mamba':
+            N = 16
+            inputs = (randn(B, D, T), randn(B, D, T), randn(D), randn(D, N), randn(B, N, T), randn(B, N, T))
+            st = jit('step', ops.mamba)
+
+            def layer(u, dt, dt_bias, A_log, b, c):
+                dt = F.softplus(dt + dt_bias[:, None])
+                A = -A_log.exp()
+                u, dt, b, c = [i.mT[:, :, None, :, None] for i in (u, dt, b, c)]
+                s = th.zeros(B, 1, D, N, device=u.device, dtype=u.dtype)
+                return st(u, dt, A[None, None, None], b.mT, c.mT, s)[0].squeeze(2).mT
+        else:
+            inputs = (randn(B, T, D), randn(B, T, D))
+            st = jit('step', ops.hgrn)
+
+            def layer(x, gate):
+                f = th.sigmoid(gate)
+                x, gate = (1 - f) * x, -F.softplus(-gate)       # input gate tied to the forget gate, whose log drives the state
+                s = th.zeros(B, 1, D, 1, device=x.device, dtype=x.dtype)
+                x, gate = [i[:, :, None, :, None] for i in (x, gate)]
+                return st(x, gate, s)[0].squeeze(2)
+        return inputs, layer, steps
 
     if op == 'rwkv7':
         r, w, k, v, a, b = [randn(B, T, H, C) for _ in range(6)]
@@ -192,12 +277,17 @@ def main(argv=None):
     ap.add_argument('--check-flex', action='store_true')
     ap.add_argument('--torch-compile', action='store_true')
     ap.add_argument('--forward', action='store_true', help='forward pass only')
+    ap.add_argument('--raw', action='store_true', help='the layer takes raw projections and prepares them itself (ops: ' + ', '.join(RAW_OPS) + ')')
+    ap.add_argument('--fuse', action='store_true', help='run the layer through flex_rnn_amd.layer (input preparation moves into the step)')
     a = ap.parse_args(argv)
     check = a.check_flex or not a.benchmark_flex
     D = a.modeldim or (256 if check else 4096)
     T = a.seqlen or (256 if check else 1024)
     print(f'Testing {a.op}\nInput sizes B={a.batchsz}, T={T}, H={D // a.headsz}, C={a.headsz}')
-    inputs, layer, steps = build(a.op, a.batchsz, T, D, a.headsz, 'cuda')
+    inputs, layer, steps = build(a.op, a.batchsz, T, D, a.headsz, 'cuda', raw=a.raw)
+    eager_layer = layer
+    if a.fuse:
+        layer = flex_rnn_amd.layer(layer)
     if not check:
         if a.op not in ('s4d', 'mamba'):
             inputs = tuple(i.to(th.bfloat16) for i in inputs)
@@ -211,7 +301,7 @@ def main(argv=None):
         for s in steps.values():
             s.apply = s.naive_fp64
         try:
-            return layer(*args)
+            return eager_layer(*args)
         finally:
             for k, s in steps.items():
                 s.apply = saved[k]

@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import inspect
 import uuid
+import weakref
 
 import torch as th
 
@@ -34,6 +35,14 @@ def _sig(tensors):
 
 
 class jit:
+    _instances = weakref.WeakValueDictionary()      # dispatcher name of the forward operator -> its jit object
+
+    @classmethod
+    def instance_of(cls, op_name: str):
+        """The jit object whose forward operator has this dispatcher name (`flex_rnn::fw_<id>`, with or without an
+        overload suffix), or None: lets a traced graph be mapped back to the objects it calls."""
+        return cls._instances.get(op_name.split('.')[0])
+
     def __init__(self, step, n_step_args=None, dynamic=False):
         self.step = step
         self.forward_func = self.backward_func = None
@@ -235,6 +244,7 @@ class jit:
 
         apply.register_autograd(backward, setup_context=setup_context)
         self._fw_op, self._bw_op = apply, backward_inner
+        jit._instances['flex_rnn::fw_' + uid] = self
         return lambda *args: apply(*args)[:nout + nst]
 
 

@@ -151,6 +151,17 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
         else:
             bsum_n.append(n.name)
 
+    # A forward sum without a row extent (the squared norm of a key that the step normalises, say) depends on a
+    # timestep's row / scalar inputs only - anything that reads the state varies along rows.  It is not saved per state
+    # row like the others: every kernel forms it again from the inputs, once per timestep.
+    jext = joint.ext_table()
+    aux_all = [a for a in aux_all if jext[a][0]]
+
+    def row_sums(g: Graph):
+        """Sums in `g` over an operand that varies along rows: those a per-element pass cannot contain."""
+        gm = g.ext_table()
+        return [n.name for n in g.nodes if n.op == 'sum' and gm[n.args[0]][0]]
+
     mdep = {i: False for i in joint.inputs}
     for n in joint.nodes:
         mdep[n.name] = (n.name in msum_all) or any(mdep[a] for a in n.value_args())
@@ -200,7 +211,7 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
         if mdep.get(v, False):
             raise PartitionError('state / column / matrix gradient depends on a reduction over the row axis')
     drow = joint.extract('drow', drow_outs, cut=set(aux_all) | set(bsum_n))
-    if any(n.op == 'sum' for n in drow.nodes):
+    if row_sums(drow):
         raise PartitionError('unsupported reduction in the backward pass')
     daux = [s for s in bsum_n if drow.uses(s)]
 
@@ -214,7 +225,7 @@ def partition(joint: Graph, ninputs: int, nstates: int, noutputs: int,
 
     # --- restep -------------------------------------------------------------------------
     restep = joint.extract('restep', list(nst_names), cut=set(aux_all))
-    if any(n.op == 'sum' for n in restep.nodes):
+    if row_sums(restep):
         raise PartitionError('unsupported reduction while recomputing the state')
 
     aux = [a for a in aux_all if restep.uses(a) or dstep.uses(a) or drow.uses(a) or epi.uses(a)]

@@ -3,6 +3,10 @@ import sys
 
 import pytest
 
+# every launch the tests make is audited first (tensor shapes, element types and storage bounds against what the
+# kernel indexes; grid against the plan): read by flex_rnn_amd.launch when it is imported
+os.environ.setdefault('FLEX_RNN_CHECK', '1')
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -43,6 +43,29 @@ def main():
         step, spec, nst, src = cases.random_step(int(name[4:]))
         print(src)
         step, xs, ss = cases.make_inputs('gen', *dims, dtype=dtype, table={'gen': (step, spec, nst)})
+    elif name.startswith('layer:'):
+        # the step a traced layer runs instead of the user's (flex_rnn_amd.layer: input preparation moved into the step),
+        # on the raw tensors the rewritten layer hands it
+        import flex_rnn_amd
+        from flex_rnn_amd import examples
+        B, T, H, M, N = dims
+        assert M == N or name[6:] in ('mamba', 'hgrn')
+        inputs, layer, _ = examples.build(name[6:], B, T, H * M, M, 'cpu', raw=True)
+        inputs = [i.to(dtype) for i in inputs]
+        lay = flex_rnn_amd.layer(layer)
+        lay.graph(*inputs)
+        call, = lay.calls
+        seen = {}
+
+        def capture(*a):
+            seen['args'] = a
+            return call.fused.naive(*a)
+
+        call.fused.apply = capture
+        lay(*inputs)
+        step = call.fused.step
+        xs, ss = list(seen['args'][:call.fused.ninputs]), list(seen['args'][call.fused.ninputs:])
+        ss = [(th.randn(s.shape, generator=th.Generator().manual_seed(4)) * 0.3).to(dtype) for s in ss]
     elif name.startswith('cfg:'):
         wl = configs.make(name[4:], dims=dims, dtype=dtype)
         step, xs, ss = wl.step, wl.inputs, wl.states

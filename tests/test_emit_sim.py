@@ -65,6 +65,12 @@ RUNS = [
     # a single state row (M = 1), down to a scalar state (M = N = 1)
     ('mlstm_gates', '2,8,2,1,1', 'f32', 1),
     ('gla', '2,8,2,1,16', 'f32', 0),
+    # steps built by `flex_rnn_amd.layer`: the layer's input preparation (softplus / sigmoid gates, L2-normalised keys,
+    # a gate tied to another) evaluated inside the kernels, gradients with respect to the raw projections
+    ('layer:rwkv7', '2,19,2,16,16', 'f32', 1),
+    ('layer:gated_delta_rule', '1,16,2,32,32', 'bf16', 0),
+    ('layer:mamba2', '2,21,2,16,16', 'f32', 1),
+    ('layer:hgrn', '2,9,1,32,1', 'f32', 0),
 ]
 
 
@@ -121,6 +127,34 @@ def test_tile_overrides(case, dims, dtype, end, tile):
     r = subprocess.run([sys.executable, RUNNER, case, dims, dtype, str(end)], capture_output=True, text=True, timeout=900, env=env)
     assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
     assert tile.split(',')[0] in r.stdout.replace(' ', '')
+
+
+# The hardened harness: threads of a workgroup resumed in a fresh random order in every barrier phase and workgroups
+# shuffled (a missing barrier, a read of LDS before its write or a dependence on the order of workgroups then shows
+# for some seed), LDS poisoned with NaNs at the start of every workgroup, every uninitialised local variable a NaN
+# pattern, array-bounds checks on registers and LDS, guard regions of 1 GiB around every tensor, the product's launch
+# audit on.  The first rows are the shape of the one GPU memory fault on record (bf16, a partial last chunk, row inputs
+# shared over heads), with default knobs and with the deferred flush; `all` runs every candidate build the first call
+# would time on a GPU through the product's own choice logic (`CompiledPlan._tune` / `_select`).
+HARDENED = [
+    ('cfg:mamba2', '2,19,4,64,128', 'bf16', 1, '', 1, False),
+    ('cfg:mamba2', '2,19,4,64,128', 'bf16', 0, 'DF=1', 2, False),
+    ('cfg:mamba2', '2,19,2,16,128', 'bf16', 1, 'DF=1', 3, True),
+    ('cfg:mamba2', '2,19,2,16,128', 'bf16', 0, '', 4, True),
+    ('cfg:rwkv7', '1,21,1,32,128', 'bf16', 1, '', 5, False),
+    ('cfg:mamba1', '2,13,2,64,16', 'f32', 0, '', 6, False),
+    ('cfg:gated_delta_rule', '1,19,2,32,128', 'bf16', 1, 'DF=1', 7, False),
+]
+
+
+@pytest.mark.parametrize('case,dims,dtype,end,tile,seed,every', HARDENED)
+def test_hardened_harness(case, dims, dtype, end, tile, seed, every):
+    env = dict(os.environ, FLEX_RNN_TILE=tile, HIPSIM_SEED=str(seed), HIPSIM_UNINIT='1', HIPSIM_BOUNDS='1',
+               HIPSIM_CANDIDATES='1' if every else '0', FLEX_RNN_CHECK='1')
+    r = subprocess.run([sys.executable, RUNNER, case, dims, dtype, str(end)], capture_output=True, text=True, timeout=1500, env=env)
+    assert r.returncode == 0, f'rc={r.returncode}\n{r.stdout[-2000:]}\n{r.stderr[-3000:]}'
+    if every:
+        assert 'frnn_fw#1' in r.stdout and 'frnn_bw1#1' in r.stdout and 'frnn_bw2#1' in r.stdout, r.stdout[-600:]
 
 
 @pytest.mark.parametrize('case,dims', [('rwkv7', '3,32,2,16,16'), ('cfg:mamba1', '2,16,4,32,16')])

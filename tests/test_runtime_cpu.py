@@ -224,3 +224,57 @@ def test_static_scratch_launch_validates_before_touching_the_device(runtime_lib,
     ''')
     r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
     assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr
+
+
+def test_launch_audit_rejects_what_the_kernels_take_on_trust(runtime_lib, tmp_path):
+    """FLEX_RNN_CHECK=1: before a launch, every tensor must have the shape and element type the kernel's index
+    arithmetic was emitted for, hidden buffers must be contiguous, and the grid must cover the plan.  Runs the real
+    host path (planned, compiled and loaded kernels; the stand-in HIP answers the module calls) up to the launch."""
+    so = tmp_path / 'libfakehip.so'
+    subprocess.run(['g++', '-shared', '-fPIC', '-o', str(so), os.path.join(ROOT, 'tests', 'fakehip', 'fakehip.cpp')], check=True)
+    code = textwrap.dedent(f'''
+        import ctypes, os, sys
+        os.environ['FLEX_RNN_CHECK'] = '1'
+        os.environ['FLEX_RNN_TUNE'] = '0'
+        sys.path.insert(0, {ROOT!r}); sys.path.insert(0, os.path.join({ROOT!r}, 'tests'))
+        fake = ctypes.CDLL({str(so)!r}, mode=ctypes.RTLD_GLOBAL)
+        import torch as th
+        import cases
+        from flex_rnn_amd import planner, launch
+        step, xs, ss = cases.make_inputs('gla', 2, 16, 2, 16, 16, dtype=th.float32)
+        plan, fm, bm = planner.make_plan(step, xs, ss)
+        class OnHost(launch.CompiledPlan):
+            _on_gpu = False
+        cp = OnHost(plan)
+        B, T, H, M, N = 2, 16, 2, 16, 16
+        good = {{'aux': th.empty(len(plan.part.aux), B, H, T, M), 'out0': th.empty(B, T, H, M), 'st0': ss[0], 'stT0': th.empty_like(ss[0]),
+                'sck0': th.empty(B, H, plan.nchunks, M, plan.NP)}}
+        for i, x in enumerate(xs):
+            good[f'in{{i}}'] = x
+        buf, _ = cp._pack('frnn_fw', good)
+        assert len(buf) == cp.kernels['frnn_fw'][1].arg_bytes
+        def refused(change, msg):
+            bad = dict(good); bad.update(change)
+            try:
+                cp._pack('frnn_fw', bad)
+            except AssertionError as e:
+                assert msg in str(e), (msg, str(e))
+            else:
+                raise SystemExit('accepted ' + str({{k: tuple(v.shape) for k, v in change.items()}}))
+        refused({{'out0': th.empty(B, T - 1, H, M)}}, 'the kernel indexes')
+        refused({{'sck0': th.empty(B, H, plan.nchunks - 1 or 2, M, plan.NP)}}, 'the kernel indexes')
+        refused({{'in0': xs[0].to(th.bfloat16)}}, 'was emitted for')
+        refused({{'sck0': th.empty(B, H, plan.nchunks, plan.NP, M).transpose(-1, -2)}}, 'must be contiguous')
+        refused({{'st0': ss[0][:, :1]}}, 'the kernel indexes')
+        try:
+            cp._pack('frnn_fw', {{k: v for k, v in good.items() if k != 'out0'}})
+        except AssertionError as e:
+            assert 'takes a tensor called out0' in str(e), e
+        else:
+            raise SystemExit('packed without out0')
+        cp._grid['frnn_fw'] = (cp._grid['frnn_fw'][0] + 1,) + cp._grid['frnn_fw'][1:]
+        refused({{}}, 'does not cover')
+        print('ok')
+    ''')
+    r = subprocess.run([sys.executable, '-c', code], capture_output=True, text=True)
+    assert r.returncode == 0 and 'ok' in r.stdout, r.stdout + r.stderr

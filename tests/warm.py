@@ -78,6 +78,11 @@ def example_plans():
             a = EXAMPLE_ARGS
             inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta')
             layer(*inputs)
+        # tests/test_gpu_layer.py: the same layers traced by `flex_rnn_amd.layer` (plans of the fused steps included)
+        for op, raw, dtype in [(op, False, th.float32) for op in examples.OPS] + \
+                [(op, True, dt) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)]:
+            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta', raw=raw)
+            flex_rnn_amd.layer(layer).graph(*[i.to(dtype) for i in inputs])
     finally:
         jit_mod.build_twopass = orig
     return plans
