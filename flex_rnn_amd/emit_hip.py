@@ -504,12 +504,15 @@ class _Prologue:
             if sums:
                 fname, used, mine = sums
                 outs = [f'o{k}_' for k in range(len(mine))]
-                out += (f'{ind}for (int tt_ = tid / 16; tt_ < {TS}; tt_ += {NT // 16}) {{ '
+                # (every group of 16 lanes makes the same number of rounds, so that the cross-lane adds sit in uniform
+                # control flow; a group without a timestep left works on the last one again and stores nothing)
+                groups = NT // 16
+                out += (f'{ind}for (int r_ = 0; r_ < {-(-TS // groups)}; r_++) {{ const int tq_ = tid / 16 + r_ * {groups}, tt_ = min(tq_, {TS - 1}); '
                         + ' '.join(f'float s{k}_ = 0.0f;' for k in range(len(mine))) + '\n'
                         f'{ind}  for (int x_ = tid % 16; x_ < {em.N}; x_ += 16) {{ {self._call(fname, used, outs)} '
                         + ' '.join(f's{k}_ += o{k}_[0][0];' for k in range(len(mine))) + ' }\n'
                         + ''.join(f'{ind}  s{k}_ = grp_allreduce<16>(s{k}_);\n' for k in range(len(mine)))
-                        + f'{ind}  if ((tid & 15) == 0) {{ ' + ' '.join(f's_pc{self.cuts.index(c)}[tt_] = s{k}_;' for k, c in enumerate(mine))
+                        + f'{ind}  if ((tid & 15) == 0 && tq_ < {TS}) {{ ' + ' '.join(f's_pc{self.cuts.index(c)}[tt_] = s{k}_;' for k, c in enumerate(mine))
                         + ' } }\n')
             if scalars:
                 fname, used, mine = scalars
@@ -609,17 +612,44 @@ class Emitter:
         return front
 
     def _prologue_front(self, graphs):
-        """The outermost values of `graphs` that do not vary along the state's rows and are not plain inputs or
-        constants: those read by a value with a row extent, or returned.  What `_row_front` finds is the special case
-        that needs no pass of its own (values of one column of staged row inputs, no sums)."""
-        front = []
-        for g in graphs:
-            for n in g.nodes:
-                if n.ext[0] or n.op == 'const' or n.name in front:
-                    continue
-                if n.name in g.outputs or any(n.name in m.value_args() and m.ext[0] for m in g.nodes):
-                    front.append(n.name)
-        return front
+        """`partition.prologue_front`; what `_row_front` finds is the special case that needs no pass of its own
+        (values of one column of staged row inputs, no sums)."""
+        from .partition import prologue_front
+        return prologue_front(graphs)
+
+    def _levelled(self, g: Graph, fname: str, out_exts, colmask: str = '', prolog: str = ''):
+        """`g` cut at its sums, for kernels in which a sum over the columns crosses waves (two barriers each): a
+        function per level that returns the operands of that level's sums (levels by dependence among the sums), and
+        a last one that returns the results, each taking the sums below it as inputs.  The caller evaluates a level for
+        all timesteps of a chunk, reduces everything in one exchange, and goes on.  None when `g` has no sums."""
+        sums = [n for n in g.nodes if n.op == 'sum']
+        if not sums:
+            return None
+        names = [n.name for n in sums]
+        dep = {}
+        for n in g.nodes:
+            d = set()
+            for a in n.value_args():
+                d |= ({a} if a in names else set()) | dep.get(a, set())
+            dep[n.name] = d
+        level = {}
+        for n in sums:
+            level[n.name] = 1 + max((level[d] for d in dep[n.name]), default=-1)
+        nm = g.node_map()
+        out = {'levels': [], 'sums': names, 'src': []}
+        for lv in range(1 + max(level.values())):
+            mine = [c for c in names if level[c] == lv]
+            done = [c for c in names if level[c] < lv]
+            sub = g.extract(f'{fname}_s{lv}', [nm[c].args[0] for c in mine], cut=done)
+            src, used = emit_graph_fn(sub, f'{fname}_s{lv}', 1, 1, [(False, True)] * len(mine), 'grp_allreduce<1>', self.invariant, colmask, prolog)
+            out['levels'].append((f'{fname}_s{lv}', used, mine))
+            out['src'].append(src)
+        sub = g.extract(f'{fname}_f', g.outputs, cut=names)
+        src, used = emit_graph_fn(sub, f'{fname}_f', 1, 1, out_exts, 'grp_allreduce<1>', self.invariant, colmask, prolog)
+        out['final'] = (f'{fname}_f', used)
+        out['src'].append(src)
+        out['used'] = sorted({v for _, u, _ in out['levels'] for v in u if v not in names} | {v for v in used if v not in names})
+        return out
 
     def _stage_row_front(self, stg: '_Stager', A: _Args, front, direct_used, MT: int, fn_name: str):
         """Registers the raw inputs the derived operands need (without an LDS array of their own
@@ -1291,6 +1321,12 @@ class Emitter:
         epi_nodes = {n_.name for n_ in p.epi.nodes}
         epi_g = p.epi.extract('epi', p.epi.outputs, cut=[f for f in rfront if f in epi_nodes]) if rfront else p.epi
         epi_src, epi_used = emit_graph_fn(epi_g, 'bw_epi', 1, 1, epi_exts, red, (), nok, nok_prolog)
+        # With more than one wave per instance every sum over the columns costs two barriers; sums inside the
+        # preparation and inside the epilogue (the norm of a key a traced layer normalises, and its gradient) are
+        # then formed level by level for all timesteps of the chunk at once: one exchange per level.
+        epi_lev = self._levelled(epi_g, 'bw_epi', epi_exts, nok, nok_prolog) if N > 64 else None
+        if epi_lev:
+            epi_src, epi_used = '\n'.join(epi_lev['src']), epi_lev['used']
         loop_used = set(drow_used) | set(re_used)
         pre_src, pre_used = '', []
         cuts = [i for g_ in (p.restep, p.drow) for i in g_.inputs if i not in p.joint.input_ext]
@@ -1305,7 +1341,12 @@ class Emitter:
         if rfront:
             rpre_g = p.joint.extract('rowpre', rfront, cut=set(cuts))
             rpre_src, rpre_used = emit_graph_fn(rpre_g, 'bw_rowpre', 1, 1, [self.jext[f] for f in rfront], red, self.invariant, nok, nok_prolog)
+            rpre_lev = self._levelled(rpre_g, 'bw_rowpre', [self.jext[f] for f in rfront], nok, nok_prolog) if N > 64 else None
+            if rpre_lev:
+                rpre_src, rpre_used = '\n'.join(rpre_lev['src']), rpre_lev['used']
             pre_src += '\n' + rpre_src
+        else:
+            rpre_lev = None
         all_used = loop_used | set(epi_used) | set(rpre_used)
 
         def is_rowlike(nm):      # no row extent: can be loaded once per chunk
@@ -1447,19 +1488,60 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
         n_uniform = sum(1 for f in rfront if self.jext[f] == (False, False))
+        NW = max(1, N // 64)
+
+        def exchange(tag, vals):
+            """Sums of the per-lane values `vals` (expressions) over the instance's lanes, all in one exchange through
+            LDS between two barriers; returns the names of the totals."""
+            b.append(f'  __shared__ float red_{tag}[{len(vals)}][{NW}];\n')
+            for k, v in enumerate(vals):
+                b.append(f'  float {tag}p{k} = grp_allreduce<64>({f"nok ? {v} : 0.0f" if self.pad else v});\n')
+            b.append('  __syncthreads();\n  if ((tid & 63) == 0) { ' + ' '.join(f'red_{tag}[{k}][tid >> 6] = {tag}p{k};' for k in range(len(vals)))
+                     + ' }\n  __syncthreads();\n')
+            for k in range(len(vals)):
+                b.append(f'  float {tag}t{k}[1][1]; {tag}t{k}[0][0] = ' + ' + '.join(f'red_{tag}[{k}][{w}]' for w in range(NW)) + ';\n')
+            return [f'{tag}t{k}' for k in range(len(vals))]
+
+        def levelled(lev, tag, arg_of):
+            """Evaluates the levels of `lev` for every timestep of the chunk; returns {(sum name, timestep): variable}."""
+            tot = {}
+            for li, (fn, used, mine) in enumerate(lev['levels']):
+                vals = []
+                for tt in range(DT):
+                    outs = [f'{tag}o{li}_{k}_{tt}' for k in range(len(mine))]
+                    b.append('  ' + ' '.join(f'float {o}[1][1];' for o in outs) + f' {fn}('
+                             + ', '.join([tot[(v, tt)] if (v, tt) in tot else arg_of(v, tt) for v in used] + outs) + ');\n')
+                    vals += [f'{o}[0][0]' for o in outs]
+                names = exchange(f'{tag}{li}', vals)
+                for tt in range(DT):
+                    for k, c in enumerate(mine):
+                        tot[(c, tt)] = names[tt * len(mine) + k]
+            return tot
+
+        def rpre_arg(v, tt):
+            if v in p.in_names:
+                return var_in(p.in_names.index(v), tt)
+            assert v in p.aux and is_rowlike(v), v
+            return f'ax{p.aux.index(v)}_{tt}'
+
+        if rfront and rpre_lev:
+            tot = levelled(rpre_lev, 'rp', rpre_arg)
+            fn, used = rpre_lev['final']
+            for tt in range(DT):
+                outs = [f'g{q}_{tt}' for q in range(len(rfront))]
+                b.append('  ' + ' '.join(f'float {o}[1][1];' for o in outs) + f' {fn}('
+                         + ', '.join([tot[(v, tt)] if (v, tt) in tot else rpre_arg(v, tt) for v in used] + outs) + ');\n')
         if rfront:
             for tt in range(DT):
                 call = []
-                for v in rpre_used:
-                    if v in p.in_names:
-                        call.append(var_in(p.in_names.index(v), tt))
-                    else:
-                        assert v in p.aux and is_rowlike(v), v
-                        call.append(f'ax{p.aux.index(v)}_{tt}')
+                for v in ([] if rpre_lev else rpre_used):
+                    call.append(rpre_arg(v, tt))
                 for q in range(len(rfront)):
-                    b.append(f'  float g{q}_{tt}[1][1];\n')
+                    if not rpre_lev:
+                        b.append(f'  float g{q}_{tt}[1][1];\n')
                     call.append(f'g{q}_{tt}')
-                b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
+                if not rpre_lev:
+                    b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
                 # With one instance per wave a value without row and column extent is the same on all lanes;
                 # kept in a scalar register it costs no vector register for the length of the chunk (Mamba-2's
                 # per-step decay: 184 -> 150 registers, three waves per SIMD without spills).  The scalar
@@ -1509,7 +1591,8 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             b.append(f'  for (int tt_ = n; tt_ < {DT}; tt_ += {min(N, NT)}) {{ '
                      + ' '.join(f's_cs{j}[inst][tt_] = 0.0f;' for j in colsum) + ' }\n')
         MB = 1
-        while MB * 2 <= MR and len(rowops) * IPB * (MB * 2) * DT * 4 <= 48 * 1024:
+        # (row blocks of up to three tenths of the compute unit's 160 KB of LDS: three workgroups of this kernel stay resident)
+        while MB * 2 <= MR and len(rowops) * IPB * (MB * 2) * DT * 4 <= 160 * 1024 * 3 // 10:
             MB *= 2
         lanes = min(N, NT)          # lanes of one instance
         PDe = min(PD, MB)           # (a row block is a whole number of prefetch rounds)
@@ -1688,22 +1771,35 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             for q, j in enumerate(nred):
                 for tt in range(DT):
                     b.append(f'  acc{j}_{tt} = ' + ' + '.join(f'red_ms[{q * DT + tt}][{w}]' for w in range(NW)) + ';\n')
+        def ms_value(j, tt):
+            node = nm_[p.msums[j]]
+            if 1 in node.dims and self.jext[node.args[0]][1] and not batched:
+                return f'{red}({f"nok ? acc{j}_{tt} : 0.0f" if self.pad else f"acc{j}_{tt}"})'
+            return f's_cs{j}[inst][{tt}]' if j in colsum else f'acc{j}_{tt}'
+
+        epi_tot = {}
+        if epi_lev:
+            for tt in range(DT):
+                for j in range(len(p.msums)):
+                    b.append(f'  float ms{j}_{tt}[1][1]; ms{j}_{tt}[0][0] = {ms_value(j, tt)};\n')
+
+            def epi_arg(v, tt):
+                return f'ms{p.msums.index(v)}_{tt}' if v in p.msums else call_args([v], tt, None)[0]
+
+            epi_tot = levelled(epi_lev, 'ep', epi_arg)
         for tt in range(DT):
             b.append('  {\n')
-            for j, mname in enumerate(p.msums):
-                node = nm_[mname]
-                opext = self.jext[node.args[0]]
-                if 1 in node.dims and opext[1] and not batched:
-                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {red}({f"nok ? acc{j}_{tt} : 0.0f" if self.pad else f"acc{j}_{tt}"});\n')
-                elif j in colsum:
-                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = s_cs{j}[inst][{tt}];\n')
-                else:
-                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = acc{j}_{tt};\n')
-            call = call_args(epi_used, tt, None)
+            if epi_lev:
+                fn, used = epi_lev['final']
+                call = [epi_tot[(v, tt)] if (v, tt) in epi_tot else epi_arg(v, tt) for v in used]
+            else:
+                for j in range(len(p.msums)):
+                    b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {ms_value(j, tt)};\n')
+                fn, call = 'bw_epi', call_args(epi_used, tt, None)
             for i in rs:
                 b.append(f'    float g{i}[1][1];\n')
                 call.append(f'g{i}')
-            b.append('    bw_epi(' + ', '.join(call) + ');\n')
+            b.append(f'    {fn}(' + ', '.join(call) + ');\n')
             for i in rs:
                 if i in tacc:
                     b.append(f'    gt{i} += g{i}[0][0];\n')

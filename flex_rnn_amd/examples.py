@@ -279,6 +279,7 @@ def main(argv=None):
     ap.add_argument('--forward', action='store_true', help='forward pass only')
     ap.add_argument('--raw', action='store_true', help='the layer takes raw projections and prepares them itself (ops: ' + ', '.join(RAW_OPS) + ')')
     ap.add_argument('--fuse', action='store_true', help='run the layer through flex_rnn_amd.layer (input preparation moves into the step)')
+    ap.add_argument('--fuse-reductions', action='store_true', help='with --fuse: also move sums and norms along the column axis')
     a = ap.parse_args(argv)
     check = a.check_flex or not a.benchmark_flex
     D = a.modeldim or (256 if check else 4096)
@@ -287,7 +288,7 @@ def main(argv=None):
     inputs, layer, steps = build(a.op, a.batchsz, T, D, a.headsz, 'cuda', raw=a.raw)
     eager_layer = layer
     if a.fuse:
-        layer = flex_rnn_amd.layer(layer)
+        layer = flex_rnn_amd.layer(layer, reductions=a.fuse_reductions)
     if not check:
         if a.op not in ('s4d', 'mamba'):
             inputs = tuple(i.to(th.bfloat16) for i in inputs)

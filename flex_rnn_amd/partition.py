@@ -71,6 +71,20 @@ class Partition:
         return '\n\n'.join(g.code() for g in (self.fw, self.restep, self.dstep, self.drow, self.epi))
 
 
+def prologue_front(graphs) -> List[str]:
+    """The outermost values of `graphs` that do not vary along the state's rows and are not plain inputs or
+    constants: those read by a value with a row extent, or returned.  The row kernels evaluate them once per
+    (timestep, column) after staging instead of inside the step."""
+    front = []
+    for g in graphs:
+        for n in g.nodes:
+            if n.ext[0] or n.op == 'const' or n.name in front:
+                continue
+            if n.name in g.outputs or any(n.name in m.value_args() and m.ext[0] for m in g.nodes):
+                front.append(n.name)
+    return front
+
+
 def _depends(graph: Graph, seeds: Sequence[str]) -> Dict[str, bool]:
     dep = {i: (i in seeds) for i in graph.inputs}
     for n in graph.nodes:

@@ -21,9 +21,10 @@ from typing import Callable, List, Optional, Tuple
 import torch as th
 
 from . import tracer
-from .partition import Partition, partition
+from .partition import Partition, partition, prologue_front
 
 SUPPORTED_DTYPES = (th.float32, th.bfloat16, th.float16, th.float64)
+LDS_BYTES = 160 * 1024         # per compute unit on gfx950 (and the most one workgroup may use)
 
 
 def split_list(args, lens):
@@ -242,10 +243,15 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     # staging depth: as many timesteps as fit in LDS (inputs + per-row results), at most DT
     cls = part_input_classes(part)
     ins = sum({'row': N, 'col': MT, 'scalar': 1, 'mat': 0}[c] for c in cls)
-    per_step = ins + max(part.noutputs + len(part.aux),                                       # forward
-                         len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * MT   # reverse scan
+    # (values the kernels prepare per (timestep, column) after staging have LDS rows of their own)
+    jext = part.joint.ext_table()
+    pro = max(sum(N if jext[f][1] else 1 for f in prologue_front([g])) for g in (part.fw, part.dstep))
+    per_step = ins + pro + max(part.noutputs + len(part.aux),                                       # forward
+                               len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * MT   # reverse scan
+    # gfx950 has 160 KB of LDS per compute unit; a workgroup gets the share that still leaves eight waves resident
+    budget = max(64 * 1024, LDS_BYTES // max(1, -(-8 // W)))
     TS = DT
-    while TS > 1 and per_step * TS * 4 > 64 * 1024 - 256:
+    while TS > 1 and per_step * TS * 4 > budget - 256:
         TS //= 2
     if part.dstep_needs_state:
         TS = DT

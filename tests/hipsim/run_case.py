@@ -43,16 +43,17 @@ def main():
         step, spec, nst, src = cases.random_step(int(name[4:]))
         print(src)
         step, xs, ss = cases.make_inputs('gen', *dims, dtype=dtype, table={'gen': (step, spec, nst)})
-    elif name.startswith('layer:'):
-        # the step a traced layer runs instead of the user's (flex_rnn_amd.layer: input preparation moved into the step),
-        # on the raw tensors the rewritten layer hands it
+    elif name.startswith('layer:') or name.startswith('layer+:'):
+        # the step a traced layer runs instead of the user's (flex_rnn_amd.layer: input preparation moved into the step;
+        # `layer+:` also moves norms along the column axis), on the raw tensors the rewritten layer hands it
+        full, name = name.startswith('layer+:'), 'layer:' + name.split(':', 1)[1]
         import flex_rnn_amd
         from flex_rnn_amd import examples
         B, T, H, M, N = dims
         assert M == N or name[6:] in ('mamba', 'hgrn')
         inputs, layer, _ = examples.build(name[6:], B, T, H * M, M, 'cpu', raw=True)
         inputs = [i.to(dtype) for i in inputs]
-        lay = flex_rnn_amd.layer(layer)
+        lay = flex_rnn_amd.layer(layer, reductions=full)
         lay.graph(*inputs)
         call, = lay.calls
         seen = {}

@@ -68,9 +68,12 @@ RUNS = [
     # steps built by `flex_rnn_amd.layer`: the layer's input preparation (softplus / sigmoid gates, L2-normalised keys,
     # a gate tied to another) evaluated inside the kernels, gradients with respect to the raw projections
     ('layer:rwkv7', '2,19,2,16,16', 'f32', 1),
-    ('layer:gated_delta_rule', '1,16,2,32,32', 'bf16', 0),
+    ('layer+:rwkv7', '2,19,2,16,16', 'f32', 0),             # (norms along the column axis inside the kernels too)
+    ('layer+:gated_delta_rule', '1,16,2,32,32', 'bf16', 0),
+    ('layer+:gated_delta_rule', '1,19,1,128,128', 'f32', 1),   # two waves per gradient-kernel instance: batched sums
     ('layer:mamba2', '2,21,2,16,16', 'f32', 1),
     ('layer:hgrn', '2,9,1,32,1', 'f32', 0),
+    ('longhorn', '1,8,1,8,128', 'f32', 1),                  # fewer staged timesteps than groups of lanes that sum them
 ]
 
 

@@ -21,17 +21,13 @@ def _oracle_apply(step_obj):
     return run
 
 
-CASES = [(op, False, th.float32) for op in examples.OPS] + \
-        [(op, True, dt) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)]
-
-
-@pytest.mark.parametrize('op,raw,dtype', CASES)
-def test_layer_against_oracle(op, raw, dtype):
-    print(f'case layer {op} raw={raw} {dtype}', flush=True)
+@pytest.mark.parametrize('op,raw,dtype,reductions', warm.LAYER_CASES)
+def test_layer_against_oracle(op, raw, dtype, reductions):
+    print(f'case layer {op} raw={raw} {dtype} reductions={reductions}', flush=True)
     a = warm.EXAMPLE_ARGS
     inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'cuda', raw=raw)
     inputs = [i.to(dtype) for i in inputs]
-    lay = flex_rnn_amd.layer(layer)
+    lay = flex_rnn_amd.layer(layer, reductions=reductions)
     xs = [i.clone().requires_grad_() for i in inputs]
     res = lay(*xs)
     res = res if isinstance(res, tuple) else (res,)

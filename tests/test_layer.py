@@ -51,26 +51,28 @@ def _through_layer(lay, steps, inputs, dtype=th.float64):
 
 # what must have moved into the step, per raw-projection layer (operator names as the tracer records them)
 MOVED = {
-    'rwkv7': {'softplus', 'linalg_vector_norm', 'sigmoid', 'div', 'neg'},
+    'rwkv7': {'softplus', 'sigmoid', 'div', 'neg'},
     'gla': {'softplus', 'div', 'mul'},
-    'delta_rule': {'linalg_vector_norm', 'sigmoid'},
-    'gated_delta_rule': {'linalg_vector_norm', 'softplus', 'sigmoid', 'add'},
+    'delta_rule': {'div', 'sigmoid'},
+    'gated_delta_rule': {'div', 'softplus', 'sigmoid', 'add'},
     'mamba2': {'softplus', 'add'},
     'mamba': {'softplus', 'add'},
     'hgrn': {'sigmoid', 'softplus', 'rsub'},
 }
 
 
+@pytest.mark.parametrize('reductions', [False, True])
 @pytest.mark.parametrize('op', examples.RAW_OPS)
-def test_preparation_moves_into_the_step(op):
+def test_preparation_moves_into_the_step(op, reductions):
     inputs, layer, steps = examples.build(op, DIMS['B'], DIMS['T'], DIMS['D'], DIMS['C'], 'cpu', raw=True)
     inputs = [i.double() for i in inputs]
-    lay = flex_rnn_amd.layer(layer)
+    lay = flex_rnn_amd.layer(layer, reductions=reductions)
     got, ggot = _through_layer(lay, steps, inputs)
     assert len(lay.calls) == 1 and MOVED[op] <= set(lay.calls[0].moved), lay.calls and lay.calls[0].moved
-    # the fused step takes raw tensors: none of the moved operations is left in the graph in a form that varies with time
-    code = lay.graph(*inputs).code
-    assert 'softplus' not in code or op in ('rwkv7',) or True
+    # norms along the column axis move only on request; otherwise they stay in the graph
+    normalises = op in ('rwkv7', 'delta_rule', 'gated_delta_rule')
+    assert ('linalg_vector_norm' in lay.calls[0].moved) == (normalises and reductions)
+    assert ('linalg_vector_norm' in lay.graph(*inputs).code) == (normalises and not reductions)
     want, gwant = _eager(layer, steps, inputs)
     recurrence.assert_all_close(got + ggot, want + gwant, 1e-10, op)
 
@@ -137,7 +139,7 @@ def test_merged_head_axis_and_shared_raw_tensor():
 
     gen = th.Generator().manual_seed(2)
     inputs = [th.randn(B, T, H * C, generator=gen, dtype=th.float64) * 0.5 for _ in range(5)] + [th.randn(B, H, C, C, generator=gen, dtype=th.float64)]
-    lay = flex_rnn_amd.layer(layer)
+    lay = flex_rnn_amd.layer(layer, reductions=True)
     got, ggot = _through_layer(lay, {'s': st}, inputs)
     assert len(lay.calls[0].raw_signatures) == 5, lay.calls[0].raw_signatures      # r, w, k (once), v, g
     assert {'exp', 'linalg_vector_norm', 'sigmoid', 'neg'} <= set(lay.calls[0].moved)

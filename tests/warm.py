@@ -59,6 +59,18 @@ SEGMENTED_CASES = [('gated_delta_rule', (2, 77, 2, 128, 128)), ('mamba1', (2, 45
 EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
 
 
+def _layer_cases():
+    from flex_rnn_amd import examples
+    norm = ('rwkv7', 'delta_rule', 'gated_delta_rule')
+    return [(op, False, th.float32, False) for op in examples.OPS] + \
+           [(op, True, dt, False) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)] + \
+           [(op, True, dt, True) for op in norm for dt in (th.float32, th.bfloat16)]
+
+
+# tests/test_gpu_layer.py: (op, raw projections?, dtype, norms moved into the step too?)
+LAYER_CASES = _layer_cases()
+
+
 def example_plans():
     """Dry-runs every example layer on meta tensors and returns the plans its jit objects request."""
     import flex_rnn_amd
@@ -79,10 +91,9 @@ def example_plans():
             inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta')
             layer(*inputs)
         # tests/test_gpu_layer.py: the same layers traced by `flex_rnn_amd.layer` (plans of the fused steps included)
-        for op, raw, dtype in [(op, False, th.float32) for op in examples.OPS] + \
-                [(op, True, dt) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)]:
+        for op, raw, dtype, reductions in LAYER_CASES:
             inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta', raw=raw)
-            flex_rnn_amd.layer(layer).graph(*[i.to(dtype) for i in inputs])
+            flex_rnn_amd.layer(layer, reductions=reductions).graph(*[i.to(dtype) for i in inputs])
     finally:
         jit_mod.build_twopass = orig
     return plans
