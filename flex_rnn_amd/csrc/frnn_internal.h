@@ -13,4 +13,10 @@ struct frnn_kernel_s {
 __attribute__((visibility("hidden"))) int frnn_detail_fail(int code, const char* fmt, ...)
     __attribute__((format(printf, 2, 3)));
 
+
+// hipModuleLaunchKernel as resolved at run time by frnn_rt.cpp (the HIP runtime the process already holds), or null
+// before any HIP call was made there.  frnn_static.hip, which is linked against the HIP runtime, checks that it is
+// bound to the same one.
+extern "C" __attribute__((visibility("hidden"))) void* frnn_detail_runtime_launch_symbol();
+
 #endif

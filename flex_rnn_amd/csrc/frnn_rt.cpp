@@ -174,6 +174,7 @@ struct frnn_module_s {
   void* mod;
   std::vector<char> image;   // the code object bytes; kept for the lifetime of the module
   std::vector<frnn_kernel_s*> kernels;   // handles given out by frnn_get_kernel; freed with the module
+  std::mutex mu;                         // guards `kernels`
 };
 
 namespace {
@@ -480,9 +481,17 @@ int frnn_get_kernel(frnn_module_t m, const char* name, frnn_kernel_t* out) {
   hipError_t e = h.ModuleGetFunction(&fn, m->mod, name);
   if (e != 0) return hip_fail("hipModuleGetFunction", e);
   frnn_kernel_s* k = new frnn_kernel_s{fn, explicit_arg_bytes(m->image, name)};
-  m->kernels.push_back(k);
+  {
+    std::lock_guard<std::mutex> lock(m->mu);      // (threads may fetch kernels of one module side by side)
+    m->kernels.push_back(k);
+  }
   *out = k;
   return FRNN_OK;
+}
+
+void* frnn_detail_runtime_launch_symbol() {
+  HipApi& h = hip();
+  return h.ok ? (void*)h.ModuleLaunchKernel : nullptr;
 }
 
 int frnn_kernel_arg_bytes(frnn_kernel_t k, size_t* out) {

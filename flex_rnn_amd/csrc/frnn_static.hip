@@ -1,11 +1,13 @@
 // frnn_launch_static: the launch entry point that allocates nothing (see include/frnn_rt.h).
 //
-// The hidden buffers of a launch (state checkpoints, saved row sums, fp32 gradient accumulators) are
-// placed in one file-scope device array instead of memory the caller allocated.  Every GPU has its own
+// The hidden buffers of a launch (state checkpoints, saved row sums, any zero-filled accumulator) are
+// placed in one file-scope device array instead of memory the caller allocated (which buffers is the caller's
+// choice: the Python host puts state / d-state checkpoints and the saved sums there).  Every GPU has its own
 // copy of the array at its own address; that address is asked for once per device and is what kernels,
 // fills and copies are given.  The array's name itself is only meaningful to hipGetSymbolAddress.
 #include <hip/hip_runtime.h>
 
+#include <dlfcn.h>
 #include <stdint.h>
 #include <string.h>
 
@@ -24,6 +26,7 @@ constexpr size_t kMaxSlots = 64;
 
 std::mutex g_mu;
 unsigned char* g_base[kMaxDevices];       // per device: where that GPU's copy of `scratch` lives
+bool g_checked = false;                   // the one-runtime check below has passed
 
 // 16 bytes per thread and trip; the grid is sized by the host and every thread leaves after its share
 __global__ void __launch_bounds__(256) frnn_fill_zero(uint4* p, size_t n16) {
@@ -37,6 +40,18 @@ int scratch_of_current_device(unsigned char** out) {
   if (e != hipSuccess) return frnn_detail_fail(FRNN_ERR_HIP, "hipGetDevice failed: %s (%d)", hipGetErrorString(e), (int)e);
   if (dev < 0 || dev >= kMaxDevices) return frnn_detail_fail(FRNN_ERR_ARG, "frnn_launch_static: device %d is beyond the %d supported", dev, kMaxDevices);
   std::lock_guard<std::mutex> lock(g_mu);
+  if (!g_checked) {
+    // This file is linked against the HIP runtime; the rest of the library resolves it at run time from what the
+    // process already holds.  A kernel handle made by one copy of the runtime must not be launched through another:
+    // refuse when the two bindings live in different shared objects.
+    void* theirs = frnn_detail_runtime_launch_symbol();
+    void* mine = (void*)&hipModuleLaunchKernel;
+    Dl_info a, b;
+    if (theirs && theirs != mine && dladdr(theirs, &a) && dladdr(mine, &b) && a.dli_fname && b.dli_fname && strcmp(a.dli_fname, b.dli_fname) != 0)
+      return frnn_detail_fail(FRNN_ERR_NO_HIP, "frnn_launch_static: two HIP runtimes in one process (%s and %s); load the one the "
+                              "application uses before this library", a.dli_fname, b.dli_fname);
+    g_checked = true;
+  }
   if (!g_base[dev]) {
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
@@ -97,6 +112,7 @@ extern "C" int frnn_launch_static(frnn_kernel_t k, const uint32_t grid[3], const
       // whole 16-byte words: the region starts 256-aligned, and rounding its end up stays inside the array
       const size_t n16 = (size_t)((s.bytes + 15) / 16);
       const unsigned blocks = (unsigned)(n16 / 256 + 1 < 2048 ? n16 / 256 + 1 : 2048);
+      (void)hipGetLastError();         // (an error an earlier, unrelated call left behind is not this launch's)
       hipLaunchKernelGGL(frnn_fill_zero, dim3(blocks), dim3(256), 0, st, (uint4*)p, n16);
       hipError_t e = hipGetLastError();
       if (e != hipSuccess) return frnn_detail_fail(FRNN_ERR_HIP, "frnn_launch_static: clearing region %zu failed: %s (%d)", i, hipGetErrorString(e), (int)e);

@@ -60,9 +60,59 @@ def _is_full(name: str, i: int, j: int) -> bool:
     return j < 3 and 'BTH'[j] in _SPANS[name][i]
 
 
-def warm(cases: Iterable = CASES, verbose: bool = False, force: bool = False) -> int:
+EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # the size the example layers are checked at (`python -m flex_rnn_amd.examples --check-flex`, tests)
+
+
+def _layer_cases():
+    from flex_rnn_amd import examples
+    norm = ('rwkv7', 'delta_rule', 'gated_delta_rule')
+    return [(op, False, th.float32, False) for op in examples.OPS] + \
+           [(op, True, dt, False) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)] + \
+           [(op, True, dt, True) for op in norm for dt in (th.float32, th.bfloat16)]
+
+
+# the example layers as `flex_rnn_amd.layer` traces them: (op, raw projections?, dtype, norms moved into the step too?)
+LAYER_CASES = _layer_cases()
+
+
+def example_plans():
+    """Dry-runs every example layer on meta tensors and returns the plans its jit objects request."""
+    import sys
+    import flex_rnn_amd
+    jit_mod = sys.modules['flex_rnn_amd.jit']        # (the package attribute `jit` is the class)
+    from flex_rnn_amd import examples
+    plans = []
+    orig = jit_mod.build_twopass
+
+    def capture(step, inputs, state, dryrun=False, tile=None):
+        metas = [t.to('meta') for t in inputs], [t.to('meta') for t in state]
+        plans.append(planner.make_plan(step, *metas, tile)[0])
+        return orig(step, inputs, state, dryrun=True, tile=tile)
+
+    jit_mod.build_twopass = capture
+    try:
+        for op in examples.OPS:
+            a = EXAMPLE_ARGS
+            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta')
+            layer(*inputs)
+        # the same layers traced by `flex_rnn_amd.layer` (plans of the fused steps included)
+        for op, raw, dtype, reductions in LAYER_CASES:
+            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta', raw=raw)
+            flex_rnn_amd.layer(layer, reductions=reductions).graph(*[i.to(dtype) for i in inputs])
+    finally:
+        jit_mod.build_twopass = orig
+    return plans
+
+
+def warm(cases: Iterable = CASES, verbose: bool = False, force: bool = False, examples: bool = False) -> int:
+    """Compiles the kernels of `cases`; with `examples` also those of the example layers (eager adapters and traced
+    layers) at `EXAMPLE_ARGS`."""
     cases = list(cases)
     plans = [plan_for(name, dims, dtype) for name, dims, dtype in cases]       # (tracing: one at a time)
+    if examples:
+        extra = example_plans()
+        cases += [('example layer', (pl.B, pl.T, pl.H, pl.M, pl.N), None) for pl in extra]
+        plans += extra
     seen = set()
     n = 0
     with ThreadPoolExecutor(max_workers=3) as pool:

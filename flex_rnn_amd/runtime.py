@@ -69,7 +69,9 @@ def build_library(verbose: bool = False) -> str:
     inc = os.path.join(_ROOT, 'include')
     tmp = LIB_PATH + f'.tmp{os.getpid()}'
     hipcc = os.environ.get('FRNN_HIPCC') or '/opt/rocm/bin/hipcc'
-    cmd = [hipcc, f'--offload-arch={ARCH}', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall',
+    # (no absolute run path to the toolchain's HIP runtime: the library binds to the copy the process holds, by soname)
+    rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(hipcc))), 'lib')
+    cmd = [hipcc, f'--offload-arch={ARCH}', '-O2', '-std=c++17', '-shared', '-fPIC', '-Wall', '-no-hip-rt', '-L', rocm_lib, '-lamdhip64',
            '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
            '-I', inc, '-I', os.path.join(_HERE, 'csrc'), *srcs, '-o', tmp, '-ldl', '-pthread']
     if verbose:

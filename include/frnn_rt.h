@@ -108,8 +108,11 @@ typedef struct frnn_scratch_slot {
  * not fit, is misaligned or overlaps another one of the same call is rejected with FRNN_ERR_ARG: use
  * frnn_launch with caller-allocated buffers for such sizes.  The buffer keeps what the last launch
  * left in it.  All calls on one GPU share it: calls whose kernels may overlap in time on one GPU
- * (other streams, other threads) race unless their regions are disjoint.  The first call on each
- * device looks the buffer's address up and must not be made during stream capture. */
+ * (other streams, other threads) race unless their regions are disjoint.  The buffer used is that of the
+ * calling thread's current device, which must be the device `stream` belongs to (and the one the module was
+ * loaded on).  The first call on each device looks the buffer's address up and must not be made during stream
+ * capture.  The library must share the application's HIP runtime (see the head of this file): the call fails
+ * with FRNN_ERR_NO_HIP when it finds itself bound to a second copy. */
 int frnn_launch_static(frnn_kernel_t k, const uint32_t grid[3], const uint32_t block[3],
                        uint32_t lds_bytes, void* stream, const void* args, size_t arg_bytes,
                        const frnn_scratch_slot* slots, size_t nslots);

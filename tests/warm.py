@@ -1,5 +1,5 @@
-"""Kernel-cache warm-up for the shapes the GPU tests use (called by __graft_entry__.build();
-needs no GPU)."""
+"""Kernel-cache warm-up for the shapes only the GPU tests use (called by __graft_entry__.build() after the
+package's own `flex_rnn_amd.prebuild.warm`; needs no GPU)."""
 import os
 import sys
 
@@ -56,47 +56,7 @@ SEGMENT = 32
 SEGMENTED_CASES = [('gated_delta_rule', (2, 77, 2, 128, 128)), ('mamba1', (2, 45, 4, 128, 16))]
 
 
-EXAMPLE_ARGS = dict(B=2, T=64, D=256, C=128)      # what tests/test_gpu_examples.py runs
-
-
-def _layer_cases():
-    from flex_rnn_amd import examples
-    norm = ('rwkv7', 'delta_rule', 'gated_delta_rule')
-    return [(op, False, th.float32, False) for op in examples.OPS] + \
-           [(op, True, dt, False) for op in examples.RAW_OPS for dt in (th.float32, th.bfloat16)] + \
-           [(op, True, dt, True) for op in norm for dt in (th.float32, th.bfloat16)]
-
-
-# tests/test_gpu_layer.py: (op, raw projections?, dtype, norms moved into the step too?)
-LAYER_CASES = _layer_cases()
-
-
-def example_plans():
-    """Dry-runs every example layer on meta tensors and returns the plans its jit objects request."""
-    import flex_rnn_amd
-    jit_mod = sys.modules['flex_rnn_amd.jit']        # (the package attribute `jit` is the class)
-    from flex_rnn_amd import examples
-    plans = []
-    orig = jit_mod.build_twopass
-
-    def capture(step, inputs, state, dryrun=False, tile=None):
-        metas = [t.to('meta') for t in inputs], [t.to('meta') for t in state]
-        plans.append(planner.make_plan(step, *metas, tile)[0])
-        return orig(step, inputs, state, dryrun=True, tile=tile)
-
-    jit_mod.build_twopass = capture
-    try:
-        for op in examples.OPS:
-            a = EXAMPLE_ARGS
-            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta')
-            layer(*inputs)
-        # tests/test_gpu_layer.py: the same layers traced by `flex_rnn_amd.layer` (plans of the fused steps included)
-        for op, raw, dtype, reductions in LAYER_CASES:
-            inputs, layer, steps = examples.build(op, a['B'], a['T'], a['D'], a['C'], 'meta', raw=raw)
-            flex_rnn_amd.layer(layer, reductions=reductions).graph(*[i.to(dtype) for i in inputs])
-    finally:
-        jit_mod.build_twopass = orig
-    return plans
+EXAMPLE_ARGS, LAYER_CASES, example_plans = prebuild.EXAMPLE_ARGS, prebuild.LAYER_CASES, prebuild.example_plans
 
 
 GOLDEN = {'delta_rule': (1, 6, 2, 4, 4), 'mamba1': (2, 6, 2, 4, 4), 'mamba2': (2, 6, 2, 4, 8),
@@ -106,7 +66,7 @@ GOLDEN = {'delta_rule': (1, 6, 2, 4, 4), 'mamba1': (2, 6, 2, 4, 4), 'mamba2': (2
 def warm(force=False, seen=None):
     from flex_rnn_amd import runtime
     runtime.compile_kernel('probe', NO_ALLOC_PROBE, force=force)
-    plans = example_plans()
+    plans = []          # (the example layers' kernels are built by flex_rnn_amd.prebuild.warm(examples=True))
     for name, dims, knobs in KNOB_CASES:
         old = os.environ.get('FLEX_RNN_TILE')
         os.environ['FLEX_RNN_TILE'] = knobs
