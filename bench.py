@@ -120,12 +120,17 @@ def measure(name, steps, warmup, traffic_records):
             return round(sum(recs[k]['read_bytes'] + recs[k]['write_bytes'] for k in kernels))
         return None
 
+    def traffic_commit(kernels):
+        recs = traffic_records.get(name, {})
+        return '/'.join(sorted({str(recs[k].get('counter_run_commit', 'unrecorded')) for k in kernels if k in recs}))
+
     traffic = traffic_of([dominant])
     hbm_gbps = w['bytes_all'] * tokens / (gpu_ms * 1e-3) / 1e9
     roofline = {
         'bound': 'valu', 'kernel': dominant, 'achieved': round(achieved, 3), 'peak': PEAK_FP32_TFLOPS,
         'unit': 'TFLOP/s', 'frac': round(achieved / PEAK_FP32_TFLOPS, 4), 'traffic': traffic,
-        'traffic_source': ('profiles/hbm_traffic.json (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this kernel build)'
+        'traffic_source': (f'stored, not measured in this run: profiles/hbm_traffic.json, rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on this '
+                           f'kernel build (cache key checked), counter run at commit {traffic_commit([dominant])}'
                            if traffic is not None else 'none: no committed counter run for the kernel build that ran'),
         'kernel_ms': {k: round(v, 4) for k, v in kavg.items()},
         'step_achieved': round(step_tflops, 3), 'step_frac': round(step_tflops / PEAK_FP32_TFLOPS, 4),

@@ -381,6 +381,13 @@ def export_shipped_picks(device_name: str, path: str = None) -> int:
     return len(have)
 
 
+def device_id(index: int) -> str:
+    """What timed choices are keyed on: the GPU's architecture and number of compute units (`gfx950-256cu`).  Not its
+    marketing name, which the driver reports differently from one tool to the next (empty under a profiler)."""
+    props = th.cuda.get_device_properties(index)
+    return f'{props.gcnArchName.split(":")[0]}-{props.multi_processor_count}cu'
+
+
 class CompiledPlan:
     _tune_pending = frozenset()
     _tune_rounds = 4            # rounds over the candidates when a kernel is timed; the first one is not counted
@@ -432,12 +439,11 @@ class CompiledPlan:
             self._install(k, v, chosen)
 
     def _device_name(self):
-        """Name of the GPU the plan is loaded on (part of the key under which timed choices are stored)."""
+        """Identity of the GPU the plan is loaded on (part of the key under which timed choices are stored)."""
         if getattr(self, '_dev_name', None) is None:
             on_gpu = self.device is not None and self.device.type == 'cuda'
             if on_gpu:
-                idx = self.device.index if self.device.index is not None else th.cuda.current_device()
-                self._dev_name = th.cuda.get_device_name(idx)
+                self._dev_name = device_id(self.device.index if self.device.index is not None else th.cuda.current_device())
             else:
                 self._dev_name = str(self.device)
         return self._dev_name
