@@ -1433,11 +1433,11 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
                     b.append(f'  float gh{i}_{tt} = 0.0f;\n')
         b.append(f'  for (int hh = 0; hh < {HB}; hh++) {{\n  const int h = h0 + hh; const int bh = b * H + h;\n')
 
-        def load_in(i, tt, m=None):
+        def load_in(i, tt, m=None, col='nc'):
             ext = self.in_ext(i)
             dt = DT_CODE[plan.in_dtypes[i]]
             idx = self._in_index(A, i, t=(tclamp(tt) if self.tdep[i] else '0'),
-                                 m=('m' if ext[0] else None), n=('nc' if ext[1] else None))
+                                 m=('m' if ext[0] else None), n=(col if ext[1] else None))
             ld = f'ldf<{dt}>({A.p(f"in{i}")}, {idx})'
             return f'(nok ? {ld} : 0.0f)' if (self.pad and ext[1]) else ld
 
@@ -1471,19 +1471,30 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
                         f'(i64)h * {A.s(nmv, 2)} + (i64)({mexpr}) * {A.s(nmv, 3)})')
             raise AssertionError(v)
 
-        # ---- per-chunk loads of everything without a row extent
-        for i in range(nin):
-            if p.in_names[i] not in all_used or self.in_ext(i)[0]:
-                continue
-            if self.tdep[i]:
-                for tt in range(DT):
-                    b.append(f'  float x{i}_{tt}[1][1]; x{i}_{tt}[0][0] = {load_in(i, tt)};\n')
-            else:
-                b.append(f'  float x{i}[1][1]; x{i}[0][0] = {load_in(i, 0)};\n')
-        for k in range(naux):
-            if p.aux[k] in all_used and is_rowlike(p.aux[k]):
-                for tt in range(DT):
-                    b.append(f'  float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "0")};\n')
+        # ---- per-chunk loads of everything without a row extent.  Inputs that only the preparation before the row loop and
+        # the epilogue read (the raw projections behind a preparation that a traced layer moved into the step) would
+        # occupy registers across the row loop, which decides the kernel's occupancy: when there are more than 32 such
+        # registers they are loaded in a block of their own for the preparation and again after the row loop (`late`).
+        # Fewer stay where they are: the second load's latency is not hidden (Mamba-2: 1.06 -> 1.13 ms when tried).
+        def chunk_loads(names, col='nc'):
+            out = []
+            for i in range(nin):
+                if p.in_names[i] not in names or self.in_ext(i)[0]:
+                    continue
+                if self.tdep[i]:
+                    for tt in range(DT):
+                        out.append(f'  float x{i}_{tt}[1][1]; x{i}_{tt}[0][0] = {load_in(i, tt, col=col)};\n')
+                else:
+                    out.append(f'  float x{i}[1][1]; x{i}[0][0] = {load_in(i, 0, col=col)};\n')
+            for k in range(naux):
+                if p.aux[k] in names and is_rowlike(p.aux[k]):
+                    for tt in range(DT):
+                        out.append(f'  float ax{k}_{tt}[1][1]; ax{k}_{tt}[0][0] = {aux_load(k, tt, "0")};\n')
+            return out
+
+        prep_only = all_used - loop_used
+        late = DT * sum(1 for i in range(nin) if p.in_names[i] in prep_only and not self.in_ext(i)[0] and self.tdep[i]) >= 32
+        b += chunk_loads(all_used & loop_used if late else all_used)
         for j in loop_ops:
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
@@ -1524,32 +1535,40 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             assert v in p.aux and is_rowlike(v), v
             return f'ax{p.aux.index(v)}_{tt}'
 
+        def uniform(tt):
+            # With one instance per wave a value without row and column extent is the same on all lanes;
+            # kept in a scalar register it costs no vector register for the length of the chunk (Mamba-2's
+            # per-step decay: 184 -> 150 registers, three waves per SIMD without spills).  The scalar
+            # inputs themselves stay in vector registers: as scalar operands of the row loop's
+            # multiply-adds they cost moves (gated delta rule: 7 % slower).
+            return [f'  g{q}_{tt}[0][0] = wave_uniform(g{q}_{tt}[0][0]);\n' for q, f in enumerate(rfront)
+                    if IPB == 1 and self.jext[f] == (False, False) and n_uniform * DT <= 32]      # (more would spill scalar registers)
+
+        if rfront and late:
+            for tt in range(DT):
+                b.append('  ' + ' '.join(f'float g{q}_{tt}[1][1];' for q in range(len(rfront))) + '\n')
+            b.append('  {\n')
+            b += chunk_loads(set(rpre_used) - loop_used)
         if rfront and rpre_lev:
             tot = levelled(rpre_lev, 'rp', rpre_arg)
             fn, used = rpre_lev['final']
             for tt in range(DT):
                 outs = [f'g{q}_{tt}' for q in range(len(rfront))]
-                b.append('  ' + ' '.join(f'float {o}[1][1];' for o in outs) + f' {fn}('
+                b.append('  ' + ('' if late else ' '.join(f'float {o}[1][1];' for o in outs)) + f' {fn}('
                          + ', '.join([tot[(v, tt)] if (v, tt) in tot else rpre_arg(v, tt) for v in used] + outs) + ');\n')
-        if rfront:
+                b += uniform(tt)
+        if rfront and not rpre_lev:
             for tt in range(DT):
-                call = []
-                for v in ([] if rpre_lev else rpre_used):
-                    call.append(rpre_arg(v, tt))
+                call = [rpre_arg(v, tt) for v in rpre_used]
                 for q in range(len(rfront)):
-                    if not rpre_lev:
+                    if not late:
                         b.append(f'  float g{q}_{tt}[1][1];\n')
                     call.append(f'g{q}_{tt}')
-                if not rpre_lev:
-                    b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
-                # With one instance per wave a value without row and column extent is the same on all lanes;
-                # kept in a scalar register it costs no vector register for the length of the chunk (Mamba-2's
-                # per-step decay: 184 -> 150 registers, three waves per SIMD without spills).  The scalar
-                # inputs themselves stay in vector registers: as scalar operands of the row loop's
-                # multiply-adds they cost moves (gated delta rule: 7 % slower).
-                for q, f in enumerate(rfront):
-                    if IPB == 1 and self.jext[f] == (False, False) and n_uniform * DT <= 32:      # (more would spill scalar registers)
-                        b.append(f'  g{q}_{tt}[0][0] = wave_uniform(g{q}_{tt}[0][0]);\n')
+                b.append('  bw_rowpre(' + ', '.join(call) + ');\n')
+                b += uniform(tt)
+        if rfront and late:
+            b.append('  }\n')
+        if rfront:
             for q in g_tables:
                 b.append(f'  __shared__ float s_g{q}[{IPB}][{DT}];\n')
                 if HB > 1:
@@ -1771,6 +1790,13 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             for q, j in enumerate(nred):
                 for tt in range(DT):
                     b.append(f'  acc{j}_{tt} = ' + ' + '.join(f'red_ms[{q * DT + tt}][{w}]' for w in range(NW)) + ';\n')
+        if late:
+            # An input the preparation has read as well is read again here through a column index the compiler cannot
+            # relate to the first one: otherwise it keeps the DT 64-bit addresses of the first read in registers
+            # for the length of the row loop (gated linear attention with its gate's raw projection: 195 -> 169).
+            b.append('  int nc_late = nc; asm volatile("" : "+v"(nc_late));\n')
+            b += chunk_loads(set(epi_used) - loop_used, col='nc_late')
+
         def ms_value(j, tt):
             node = nm_[p.msums[j]]
             if 1 in node.dims and self.jext[node.args[0]][1] and not batched:

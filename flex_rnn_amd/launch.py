@@ -151,6 +151,19 @@ def _alt_splits(plan):
     return [alt for alt in (ms // 4, ms * 4) if alt >= 2 and -(-plan.M // alt) >= 4 and alt <= 65535]
 
 
+def _prologue_nodes(joint, front) -> int:
+    """How many operations the values in `front` take to compute from the inputs (a light preparation - one product, one
+    exponential - is not worth a tile of its own)."""
+    nm, seen, stack = joint.node_map(), set(), list(front)
+    while stack:
+        v = stack.pop()
+        if v in seen or v not in nm:
+            continue
+        seen.add(v)
+        stack.extend(nm[v].value_args())
+    return sum(1 for v in seen if nm[v].op != 'const')
+
+
 def row_kernel_tiles(plan, reverse: bool):
     """(L, C, R, W) candidates for the forward kernel (or the reverse scan): the heuristic's choice
     first; half the rows per lane (more, lighter waves) with the same and with twice the waves per
@@ -166,9 +179,9 @@ def row_kernel_tiles(plan, reverse: bool):
     fixed_r = reverse and plan.part.dstep_needs_state          # one row per lane there (register budget)
     out = []
 
-    def add(L, C, r, w):
+    def add(L, C, r, w, most=8):
         G = 64 // L
-        if r >= 1 and 1 <= w <= 8 and (w == 1 or w * G * r <= max(plan.M, G * r)) and (L, C, r, w) not in out and len(out) < 5:
+        if r >= 1 and 1 <= w <= most and (w == 1 or w * G * r <= max(plan.M, G * r)) and (L, C, r, w) not in out and len(out) < 6:
             out.append((L, C, r, w))
 
     add(t.L, t.C, R, W)
@@ -182,6 +195,15 @@ def row_kernel_tiles(plan, reverse: bool):
         add(t.L // 2, t.C * 2, R, 2 * W)
     if t.L == 16 and t.C == 8 and R > 1 and not fixed_r:
         add(8, 16, R // 2, 2 * W)
+    # Values the kernel prepares once per (timestep, column) after staging (`emit_hip._Prologue`) are prepared by every
+    # workgroup of a head; where the heuristic spreads a head over several workgroups, one workgroup for the whole head (up to
+    # 16 waves, the same rows per lane) does that work once; offered when the preparation is six operations or more
+    from .partition import prologue_front
+    graphs = [plan.part.dstep] + ([plan.part.restep] if plan.part.dstep_needs_state else []) if reverse else [plan.part.fw]
+    G = 64 // t.L
+    whole = plan.M // (G * R) if plan.M % (G * R) == 0 else 0
+    if _prologue_nodes(plan.part.joint, prologue_front(graphs)) >= 6 and whole > W and whole & (whole - 1) == 0:
+        add(t.L, t.C, R, whole, most=16)
     return out
 
 

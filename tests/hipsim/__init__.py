@@ -41,6 +41,7 @@ def _compile_host(spec) -> str:
     src = spec.source.replace('#include <hip/hip_runtime.h>', '#include "hipsim.h"')
     assert 'hipsim.h' in src
     src = re.sub(r'__attribute__\(\(amdgpu_waves_per_eu\([^)]*\)\)\)', '', src)      # (an occupancy request; means nothing on the host)
+    src = src.replace('"+v"', '"+r"')      # (the register class of an empty asm statement that hides a value's origin)
     # LDS arrays start a workgroup with undefined contents: poison each one where it is declared
     src, n = _SHARED_DECL.subn(lambda m: f'__shared__ float {m.group(1)}{m.group(2)}; sim_lds_poison({m.group(1)}, sizeof({m.group(1)}));', src)
     assert n == src.count('__shared__'), 'a __shared__ declaration the harness does not recognise'
