@@ -1262,9 +1262,12 @@ class Emitter:
         return KernelSpec('frnn_bw1', source, list(A.names), NT, (f'(M + {MT - 1}) // {MT}', 'H', 'B'), {'kind': 'row', 'MT': MT})
 
     # ------------------------------------------------------------------ bw2
-    def bw2(self, waves_per_simd: int = 0, prefetch: int = 4) -> KernelSpec:
+    def bw2(self, waves_per_simd: int = 0, prefetch: int = 4, reread_scalars: bool = False) -> KernelSpec:
         """`waves_per_simd` > 0 asks the compiler to fit that many waves on a SIMD (fewer registers,
-        possibly spills); the caller compares the outcomes."""
+        possibly spills); the caller compares the outcomes.  `reread_scalars`: per-timestep scalar inputs that the
+        preparation and the epilogue read but the row loop does not are read twice instead of kept (DT registers
+        each; worth it only where that lifts the occupancy: Mamba-2 at 128 rows 178 -> 162 registers and
+        1.13 -> 0.97 ms, the gated delta rule 252 -> 236 and 2 % slower)."""
         p, plan, t = self.p, self.plan, self.tile
         N, DT = plan.NP, t.DT              # lanes cover the padded width; `nok` marks real columns
         IPB = max(1, 64 // N)
@@ -1493,8 +1496,15 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             return out
 
         prep_only = all_used - loop_used
-        late = DT * sum(1 for i in range(nin) if p.in_names[i] in prep_only and not self.in_ext(i)[0] and self.tdep[i]) >= 32
-        b += chunk_loads(all_used & loop_used if late else all_used)
+        if DT * sum(1 for i in range(nin) if p.in_names[i] in prep_only and not self.in_ext(i)[0] and self.tdep[i]) >= 32:
+            late_in = set(prep_only)
+        elif reread_scalars:
+            late_in = {v for v in set(rpre_used) & set(epi_used) - loop_used if v in p.in_names
+                       and self.in_ext(p.in_names.index(v)) == (False, False) and self.tdep[p.in_names.index(v)]}
+        else:
+            late_in = set()
+        late = bool(late_in)
+        b += chunk_loads(all_used - late_in if late else all_used)
         for j in loop_ops:
             for tt in range(DT):
                 b.append(f'  float acc{j}_{tt} = 0.0f;\n')
@@ -1513,20 +1523,37 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
                 b.append(f'  float {tag}t{k}[1][1]; {tag}t{k}[0][0] = ' + ' + '.join(f'red_{tag}[{k}][{w}]' for w in range(NW)) + ';\n')
             return [f'{tag}t{k}' for k in range(len(vals))]
 
+        fresh = [0]
+
+        def total_of(tot, v, tt, ind='  '):
+            """A new variable holding the total of sum `v` at timestep `tt`, read from where `levelled` left it."""
+            fresh[0] += 1
+            name = f'lt{fresh[0]}'
+            b.append(f'{ind}float {name}[1][1]; {name}[0][0] = {tot[(v, tt)]};\n')
+            return name
+
         def levelled(lev, tag, arg_of):
-            """Evaluates the levels of `lev` for every timestep of the chunk; returns {(sum name, timestep): variable}."""
+            """Evaluates the levels of `lev` for every timestep of the chunk; returns {(sum name, timestep): expression
+            of the total}.  A level's totals stay in LDS and are read where they are used (`total_of`), and a
+            wave's partial sums go there as they are formed: neither holds DT registers per sum."""
             tot = {}
             for li, (fn, used, mine) in enumerate(lev['levels']):
-                vals = []
+                red_ = f'red_{tag}{li}'
+                b.append(f'  __shared__ float {red_}[{DT * len(mine)}][{NW}];\n  __syncthreads();\n')
                 for tt in range(DT):
-                    outs = [f'{tag}o{li}_{k}_{tt}' for k in range(len(mine))]
-                    b.append('  ' + ' '.join(f'float {o}[1][1];' for o in outs) + f' {fn}('
-                             + ', '.join([tot[(v, tt)] if (v, tt) in tot else arg_of(v, tt) for v in used] + outs) + ');\n')
-                    vals += [f'{o}[0][0]' for o in outs]
-                names = exchange(f'{tag}{li}', vals)
+                    outs = [f'{tag}o{li}_{k}' for k in range(len(mine))]
+                    b.append('  { ' + ' '.join(f'float {o}[1][1];' for o in outs) + '\n')
+                    args = [total_of(tot, v, tt, '    ') if (v, tt) in tot else arg_of(v, tt) for v in used]
+                    b.append(f'    {fn}(' + ', '.join(args + outs) + ');\n')
+                    for k, o in enumerate(outs):
+                        v = f'{o}[0][0]'
+                        b.append(f'    {{ const float p_ = grp_allreduce<64>({f"nok ? {v} : 0.0f" if self.pad else v}); '
+                                 f'if ((tid & 63) == 0) {red_}[{tt * len(mine) + k}][tid >> 6] = p_; }}\n')
+                    b.append('  }\n')
+                b.append('  __syncthreads();\n')
                 for tt in range(DT):
                     for k, c in enumerate(mine):
-                        tot[(c, tt)] = names[tt * len(mine) + k]
+                        tot[(c, tt)] = '(' + ' + '.join(f'{red_}[{tt * len(mine) + k}][{w}]' for w in range(NW)) + ')'
             return tot
 
         def rpre_arg(v, tt):
@@ -1548,14 +1575,14 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             for tt in range(DT):
                 b.append('  ' + ' '.join(f'float g{q}_{tt}[1][1];' for q in range(len(rfront))) + '\n')
             b.append('  {\n')
-            b += chunk_loads(set(rpre_used) - loop_used)
+            b += chunk_loads(set(rpre_used) & late_in)
         if rfront and rpre_lev:
             tot = levelled(rpre_lev, 'rp', rpre_arg)
             fn, used = rpre_lev['final']
             for tt in range(DT):
                 outs = [f'g{q}_{tt}' for q in range(len(rfront))]
-                b.append('  ' + ('' if late else ' '.join(f'float {o}[1][1];' for o in outs)) + f' {fn}('
-                         + ', '.join([tot[(v, tt)] if (v, tt) in tot else rpre_arg(v, tt) for v in used] + outs) + ');\n')
+                args = [total_of(tot, v, tt) if (v, tt) in tot else rpre_arg(v, tt) for v in used]
+                b.append('  ' + ('' if late else ' '.join(f'float {o}[1][1];' for o in outs)) + f' {fn}(' + ', '.join(args + outs) + ');\n')
                 b += uniform(tt)
         if rfront and not rpre_lev:
             for tt in range(DT):
@@ -1795,7 +1822,7 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             # relate to the first one: otherwise it keeps the DT 64-bit addresses of the first read in registers
             # for the length of the row loop (gated linear attention with its gate's raw projection: 195 -> 169).
             b.append('  int nc_late = nc; asm volatile("" : "+v"(nc_late));\n')
-            b += chunk_loads(set(epi_used) - loop_used, col='nc_late')
+            b += chunk_loads(set(epi_used) & late_in, col='nc_late')
 
         def ms_value(j, tt):
             node = nm_[p.msums[j]]
@@ -1817,7 +1844,7 @@ template <int N_> __device__ __forceinline__ float inst_total(float x) {
             b.append('  {\n')
             if epi_lev:
                 fn, used = epi_lev['final']
-                call = [epi_tot[(v, tt)] if (v, tt) in epi_tot else epi_arg(v, tt) for v in used]
+                call = [total_of(epi_tot, v, tt, '    ') if (v, tt) in epi_tot else epi_arg(v, tt) for v in used]
             else:
                 for j in range(len(p.msums)):
                     b.append(f'    float ms{j}[1][1]; ms{j}[0][0] = {ms_value(j, tt)};\n')

@@ -101,6 +101,12 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
     for pd, res in zip(depths, plain):          # (a duplicate source was dropped: zip stops short, which is fine)
         if res is not None and res['occupancy'] < 4 and (res['occupancy'] < 2 or res['vgprs'] <= 224):
             more.append(em.bw2(waves_per_simd=res['occupancy'] + 1, prefetch=pd))
+    # scalar inputs read twice instead of kept across the row loop: a candidate only where the compiler then fits more
+    # waves on a SIMD without spilling than any plain build does (elsewhere the second read just costs its latency)
+    first = len(cands)
+    add([em.bw2(prefetch=pd, reread_scalars=True) for pd in depths], optional=True)
+    best = max((res['occupancy'] for res in plain if res is not None and res['scratch'] == 0), default=0)
+    cands[first:] = [c for c in cands[first:] if c[2] is not None and c[2]['scratch'] == 0 and c[2]['occupancy'] > best]
     add(more, optional=True)
 
     def rank(c):
@@ -127,10 +133,10 @@ def gradient_kernel_builds(plan, force: bool = False, seen=None):
 
 def gradient_kernel_specs(plan, waves_per_simd: int = 0):
     """The candidate sources of the gradient kernel that do not depend on a compiler report: 4 and 2 checkpoint rows
-    in flight and, with split rows, a quarter and four times as many splits (what `gradient_kernel_builds` makes,
+    in flight, each also with scalar inputs read twice, and, with split rows, a quarter and four times as many splits (what `gradient_kernel_builds` makes,
     less the occupancy requests).  Nothing is compiled."""
     em = Emitter(plan)
-    specs = [em.bw2(prefetch=pd) for pd in (4, 2)]
+    specs = [em.bw2(prefetch=pd) for pd in (4, 2)] + [em.bw2(prefetch=pd, reread_scalars=True) for pd in (4, 2)]
     for alt in _alt_splits(plan):
         em_alt = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, MS=alt)))
         specs.append(em_alt.bw2(waves_per_simd=waves_per_simd, prefetch=4))
