@@ -147,6 +147,10 @@ HARDENED = [
     ('cfg:rwkv7', '1,21,1,32,128', 'bf16', 1, '', 5, False),
     ('cfg:mamba1', '2,13,2,64,16', 'f32', 0, '', 6, False),
     ('cfg:gated_delta_rule', '1,19,2,32,128', 'bf16', 1, 'DF=1', 7, False),
+    # traced layers at two waves per gradient-kernel instance: sums inside preparation and epilogue kept in LDS,
+    # raw projections loaded where they are used
+    ('layer+:gated_delta_rule', '1,19,1,128,128', 'bf16', 1, '', 8, False),
+    ('layer:mamba2', '1,19,2,128,128', 'bf16', 0, '', 9, False),
 ]
 
 
