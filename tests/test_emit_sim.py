@@ -117,7 +117,7 @@ TILED = [
     ('cfg:mamba2', '1,21,2,64,128', 'bf16', 0, 'DF=1,NB=3'),
     ('cfg:gated_delta_rule', '1,1,2,128,128', 'bf16', 1, 'DF=1'),
     ('cfg:gated_delta_rule', '1,9,1,16,80', 'f32', 0, 'DF=1'),
-    ('cfg:gated_delta_rule', '1,100,2,128,128', 'bf16', 1, 'DF=1,NB=0'),
+    ('cfg:gated_delta_rule', '1,68,1,128,128', 'bf16', 1, 'DF=1,NB=0'),
     ('rwkv4', '2,11,1,32,1', 'f32', 0, 'DF=1'),
     ('s4d', '2,8,1,8,6', 'f32', 1, 'DF=1'),
 ]
