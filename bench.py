@@ -170,9 +170,9 @@ def measure(name, steps, warmup, traffic_records):
     # candidate builds of each kernel as timed on the first call of this device (the fastest runs; the choice is kept
     # beside the kernel cache, so a later process reports the stored timings)
     def knobs(t, rev):
-        return [t.L, t.C, t.R1 or t.R if rev else t.R, t.W1 or t.W if rev else t.W, bool(t.NB & (2 if rev else 1)), t.UR, bool(t.DF), t.WN]
+        return [t.L, t.C, t.R1 or t.R if rev else t.R, t.W1 or t.W if rev else t.W, bool(t.NB & (2 if rev else 1)), t.UR, bool(t.DF), t.WN, bool(t.KS & (2 if rev else 1))]
 
-    res['row_kernel_builds'] = {k: {'candidates (L, C, R, W, branch-free sums, unroll, deferred flush, min waves per SIMD)':
+    res['row_kernel_builds'] = {k: {'candidates (L, C, R, W, branch-free sums, unroll, deferred flush, min waves per SIMD, row sums kept per block)':
                                     [knobs(t_, k == 'frnn_bw1') for t_ in launch.row_kernel_variants(compiled.plan, k == 'frnn_bw1')],
                                     'ms': compiled.build_times.get(k) and [finite(v) for v in compiled.build_times[k]],
                                     'ms_source': compiled.build_source.get(k, 'not timed: one candidate, or timing switched off')}

@@ -96,6 +96,9 @@ class TileConfig:
     DF: int = 0          # row kernels: 1 = a chunk's results leave LDS during the next chunk (double buffer) and checkpoints are
                          # stored after the wait for the staged operands, so that a wave's stores have a chunk's time to complete
                          # before it next waits for its prefetched loads.  Pays on some recurrences only; a timed candidate.
+    KS: int = 0          # row kernels: a block's row sums stay in registers (lane l of a group keeps the steps l, l + L, ...) and
+                         # go to LDS once per block instead of once per step, where a group has at least TS / 2 lanes: bit 0 =
+                         # forward kernel, bit 1 = reverse scan.  Fewer LDS stores for a few more vector instructions; a timed candidate.
     SH: int = 1          # reverse scan with state recompute: per-row operands loaded once for recompute and d-step
                          # (measured on RWKV-7: within 2 % of 0 either way; kept as a tuning knob)
 
@@ -247,7 +250,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
     jext = part.joint.ext_table()
     pro = max(sum(N if jext[f][1] else 1 for f in prologue_front([g])) for g in (part.fw, part.dstep))
     per_step = ins + pro + max(part.noutputs + len(part.aux),                                       # forward
-                               len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * MT   # reverse scan
+                               len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * (MT + 4)   # reverse scan (+ padding of kept row sums)
     # gfx950 has 160 KB of LDS per compute unit; a workgroup gets the share that still leaves eight waves resident
     budget = max(64 * 1024, LDS_BYTES // max(1, -(-8 // W)))
     TS = DT

@@ -120,6 +120,15 @@ TILED = [
     ('cfg:gated_delta_rule', '1,68,1,128,128', 'bf16', 1, 'DF=1,NB=0'),
     ('rwkv4', '2,11,1,32,1', 'f32', 0, 'DF=1'),
     ('s4d', '2,8,1,8,6', 'f32', 1, 'DF=1'),
+    # a block's row sums kept in registers and stored once: groups of 64, 16 and 8 lanes (one and two kept steps per lane),
+    # partial last block, double-buffered results, the reverse scan with state recompute, padded width, a tile that cannot
+    ('cfg:rwkv7', '1,37,1,128,128', 'f32', 0, 'KS=3'),
+    ('cfg:rwkv7', '1,19,2,128,128', 'bf16', 1, 'KS=3,L=8,C=16,R=2,W=8,R1=2,W1=8'),
+    ('cfg:mamba2', '1,21,2,64,128', 'bf16', 1, 'KS=3,DF=1,L=16,C=8'),
+    ('cfg:gated_delta_rule', '1,9,1,16,80', 'f32', 0, 'KS=3,L=16,C=8'),
+    ('cfg:mamba1', '2,13,2,128,16', 'f32', 1, 'KS=3,L=8,C=2'),
+    ('cfg:mamba1', '2,13,2,128,16', 'f32', 0, 'KS=3'),
+    ('mlstm_gates', '2,11,2,16,1', 'f32', 1, 'KS=3'),
 ]
 
 
