@@ -691,8 +691,8 @@ class CompiledPlan:
 
     def _tune(self, name, tensors, accumulators=()):
         """Times every candidate build of kernel `name` on the tensors of this call (one untimed
-        run, then the fastest of three timed ones, in rounds over the candidates) and keeps the
-        fastest.  The kernels only store and
+        run, then the fastest of three timed ones, in rounds over the candidates; candidates within 3 % of the
+        fastest then run again by themselves and are ranked by their medians) and keeps the fastest.  The kernels only store and
         accumulate; `accumulators` (what they add into) are put back afterwards.  Synchronises,
         once per kernel and plan; skipped while the stream is being captured."""
         if name not in self._tune_pending or self._capturing():
@@ -724,6 +724,18 @@ class CompiledPlan:
                     if i == 0:
                         raise                   # the first-ranked build must be launchable
                     usable[i] = False           # (a candidate the device refuses to launch is just not taken)
+        # a choice within 3 % is decided on more samples: the contenders alone, twice as many rounds, by their medians
+        # (the stored choice outlives this process, and the fastest of three runs favours whoever got a lucky one)
+        floor = min(times)
+        close = [i for i in range(n) if usable[i] and times[i] <= 1.03 * floor]
+        if len(close) > 1 and floor > 0.0:
+            samples = {i: [] for i in close}
+            for rnd in range(2 * self._tune_rounds):
+                for i in close:
+                    self._select(name, i)
+                    samples[i].append(self._timed_launch(name, tensors))
+            for i in close:
+                times[i] = sorted(samples[i])[len(samples[i]) // 2]
         best = min(range(len(times)), key=times.__getitem__)
         self._select(name, best)
         self.build_times[name] = times
