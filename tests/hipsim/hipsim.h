@@ -204,6 +204,7 @@ template <class T> static inline T sim_atomic_fetch_add(T* p, T v, int, int) {
 // ------------------------------------------------------------------ math + narrow floats
 #define __expf(x) expf(x)
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
+#define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __logf(x) logf(x)
 #define __log2f(x) log2f(x)
 static inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
