@@ -235,12 +235,17 @@ def row_kernel_variants(plan, reverse: bool):
     # A sequence with a partial last staging block gets no deferred-flush candidate: the one GPU memory fault on
     # record involved that form on such a sequence, and no cause has been shown (an explicit override still builds it,
     # for the CPU harness)
-    ts = base.DT if (reverse and plan.part.dstep_needs_state) else base.TS
-    may_defer = plan.T % ts == 0
     out = []
     for k, (L, C, r, w) in enumerate(row_kernel_tiles(plan, reverse)):
         tile = dataclasses.replace(base, L=L, C=C)
         tile = dataclasses.replace(tile, R1=r, W1=w) if reverse else dataclasses.replace(tile, R=r, W=w)
+        # a workgroup with more waves may use more of the LDS: it stages as many timesteps as then fit (a traced RWKV-7
+        # layer, ten staged rows per timestep: 8 at four waves, 16 at eight)
+        if w > ((base.W1 or base.W) if reverse else base.W):
+            from .planner import staging_depth
+            tile = dataclasses.replace(tile, TS=max(base.TS, staging_depth(plan.part, plan.N, w * (64 // L) * r, w, base.DT)))
+        ts = base.DT if (reverse and plan.part.dstep_needs_state) else tile.TS
+        may_defer = plan.T % ts == 0
         own = (base.NB, base.DF, base.UR, base.WN, base.KS)      # (the plan's own setting first)
         knobs = [own]
         if big:

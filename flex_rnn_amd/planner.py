@@ -180,6 +180,26 @@ def classify(inputs, state):
     return dims, cls, bcast
 
 
+def staging_depth(part, N: int, MT: int, W: int, DT: int) -> int:
+    """Timesteps staged through LDS at a time by a row-kernel workgroup of W waves that owns MT state rows: as many as
+    fit (inputs, prepared rows, per-row results), at most DT."""
+    cls = part_input_classes(part)
+    ins = sum({'row': N, 'col': MT, 'scalar': 1, 'mat': 0}[c] for c in cls)
+    # (values the kernels prepare per (timestep, column) after staging have LDS rows of their own)
+    jext = part.joint.ext_table()
+    pro = max(sum(N if jext[f][1] else 1 for f in prologue_front([g])) for g in (part.fw, part.dstep))
+    per_step = ins + pro + max(part.noutputs + len(part.aux),                                       # forward
+                               len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * (MT + 4)   # reverse scan (+ padding of kept row sums)
+    # gfx950 has 160 KB of LDS per compute unit; a workgroup gets the share that still leaves eight waves resident
+    budget = max(64 * 1024, LDS_BYTES // max(1, -(-8 // W)))
+    TS = DT
+    while TS > 1 and per_step * TS * 4 > budget - 256:
+        TS //= 2
+    if part.dstep_needs_state:
+        TS = DT
+    return TS
+
+
 def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None) -> TileConfig:
     """Tile heuristics (the counterpart of twopass.py:154-173, for 64-wide waves)."""
     N = 1 << (N - 1).bit_length()          # lanes and tiles cover the padded width
@@ -243,21 +263,7 @@ def choose_tiles(B, T, H, M, N, part: Partition, n_cu: int = 256, in_bcast=None)
         DT = 16
     while DT > 1 and DT > T:              # a partial last chunk is handled in the kernels
         DT //= 2
-    # staging depth: as many timesteps as fit in LDS (inputs + per-row results), at most DT
-    cls = part_input_classes(part)
-    ins = sum({'row': N, 'col': MT, 'scalar': 1, 'mat': 0}[c] for c in cls)
-    # (values the kernels prepare per (timestep, column) after staging have LDS rows of their own)
-    jext = part.joint.ext_table()
-    pro = max(sum(N if jext[f][1] else 1 for f in prologue_front([g])) for g in (part.fw, part.dstep))
-    per_step = ins + pro + max(part.noutputs + len(part.aux),                                       # forward
-                               len(part.aux) + part.noutputs + len(part.col_idx) + len(part.daux)) * (MT + 4)   # reverse scan (+ padding of kept row sums)
-    # gfx950 has 160 KB of LDS per compute unit; a workgroup gets the share that still leaves eight waves resident
-    budget = max(64 * 1024, LDS_BYTES // max(1, -(-8 // W)))
-    TS = DT
-    while TS > 1 and per_step * TS * 4 > budget - 256:
-        TS //= 2
-    if part.dstep_needs_state:
-        TS = DT
+    TS = staging_depth(part, N, MT, W, DT)
     # gradient kernel: one instance per (batch, head, chunk) walks all M rows.  When that gives the
     # chip too few waves (narrow states pack several instances into a wave), the rows are split
     # over MS instances whose row/scalar-input grads meet in fp32 atomics; needs an epilogue that
