@@ -13,7 +13,8 @@ own code.
 Environment: HIPSIM_SEED=<n> shuffles threads and workgroups (hipsim.h); HIPSIM_BOUNDS=1 checks
 every index into a declared array; HIPSIM_UNINIT=1 builds with clang and fills every uninitialised
 local variable with a NaN pattern; HIPSIM_CANDIDATES=1 makes `SimPlan` hold every candidate build
-the product would time on a GPU and run each of them once per kernel before settling on one.
+the product would time on a GPU and run each of them once per kernel before settling on one (the last; with
+FLEX_RNN_PICK="<kernel>=<index>" the named candidate alone, so that its results are the ones compared).
 """
 from __future__ import annotations
 
@@ -113,7 +114,9 @@ class SimPlan(CompiledPlan):
         if candidates:
             # every candidate build the product would time on the first call of a problem large enough to time the
             # code-generation knobs too
-            old, launch.TUNE_KNOBS_FROM = launch.TUNE_KNOBS_FROM, 0
+            old = launch.TUNE_KNOBS_FROM
+            if os.environ.get('HIPSIM_KNOBS', '1') == '1':      # (HIPSIM_KNOBS=0: the candidate list this problem size gets on a GPU)
+                launch.TUNE_KNOBS_FROM = 0
             try:
                 sets = {'frnn_fw': launch.row_kernel_specs(plan, False), 'frnn_bw1': launch.row_kernel_specs(plan, True),
                         'frnn_fwi': launch.row_kernel_specs(plan, False, save=False)}
@@ -131,11 +134,12 @@ class SimPlan(CompiledPlan):
         flat = [s_ for v in sets.values() for s_ in v]
         with ThreadPoolExecutor(max_workers=min(8, len(flat))) as pool:      # host compiler runs side by side
             list(pool.map(_compile_host, flat))
+        fixed = launch._fixed_picks()       # FLEX_RNN_PICK="frnn_fw=2": that candidate alone runs, so that its results are what is checked
         for name, specs in sets.items():
             self.builds[name] = [(s_, SimKernel(s_), None) for s_ in specs]
-            if len(specs) > 1:
+            if len(specs) > 1 and name not in fixed:
                 self._tune_pending = set(self._tune_pending) | {name}
-            self._select(name, 0)
+            self._select(name, min(fixed.get(name, 0), len(specs) - 1))
 
     def _device_name(self):
         return 'hipsim'

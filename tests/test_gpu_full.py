@@ -226,7 +226,7 @@ _OFF = pytest.mark.skip(reason='ended in a GPU memory fault (reported while the 
     pytest.param('mamba2', (2, 19, 4, 64, 128), 'DF=1,PF=1,SB=1', marks=_OFF)])
 def test_row_kernel_knobs_against_oracle(name, dims, knobs, monkeypatch):
     """The code-generation knobs of the row kernels that are timed candidates at the benchmark sizes (branch-free
-    row sums, deferred output flush, deeper unrolling), forced at small sizes with a partial last chunk: outputs,
+    row sums, row sums kept per block, deferred output flush, deeper unrolling), forced at small sizes with a partial last chunk: outputs,
     final state and all gradients against the oracle."""
     print(f'case knobs {name} {dims} {knobs}', flush=True)
     monkeypatch.setenv('FLEX_RNN_TILE', knobs)

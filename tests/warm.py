@@ -48,7 +48,9 @@ def no_alloc_tile(name, dims):
 
 
 # row-kernel code-generation knobs that the size of the test shapes would not make candidates (tests/test_gpu_full.py)
-KNOB_CASES = [('rwkv7', (2, 37, 2, 64, 64), 'DF=1,NB=3,UR=4'), ('mamba1', (2, 45, 4, 128, 16), 'DF=1,NB=3')]
+KNOB_CASES = [('rwkv7', (2, 37, 2, 64, 64), 'DF=1,NB=3,UR=4'), ('mamba1', (2, 45, 4, 128, 16), 'DF=1,NB=3'),
+              # a block's row sums kept in registers, two kept steps per lane (groups of 8 lanes)
+              ('gated_delta_rule', (2, 37, 2, 128, 128), 'KS=3,L=8,C=16')]
 
 
 # tests/test_gpu_full.py::test_segmented_call_against_oracle: sequences walked SEGMENT timesteps at a time
