@@ -18,6 +18,7 @@ FLEX_RNN_PICK="<kernel>=<index>" the named candidate alone, so that its results 
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import hashlib
 import os
@@ -91,9 +92,44 @@ class SimKernel:
         self.arg_bytes = int(getattr(self.lib, f'sim_args_size_{spec.name}')())
 
 
+@contextlib.contextmanager
+def poisoned_empty():
+    """While active, `torch.empty` / `empty_like` / `empty_strided` hand out floating-point memory filled with NaN: on a GPU
+    such memory holds whatever was there before, here fresh pages would read as zeros and hide a kernel that reads what
+    nothing has written (or leaves part of a result unwritten)."""
+    real = {n: getattr(th, n) for n in ('empty', 'empty_like', 'empty_strided')}
+
+    def wrap(fn):
+        def alloc(*a, **k):
+            t = fn(*a, **k)
+            if t.is_floating_point() and t.device.type == 'cpu' and t.numel():
+                th.as_strided(t, (t.untyped_storage().nbytes() // t.element_size(),), (1,), 0).fill_(float('nan'))
+            return t
+        return alloc
+    try:
+        for n, fn in real.items():
+            setattr(th, n, wrap(fn))
+        yield
+    finally:
+        for n, fn in real.items():
+            setattr(th, n, fn)
+
+
 class SimPlan(CompiledPlan):
     _on_gpu = False
     _tune_rounds = 2
+
+    def forward(self, *a, **k):
+        with poisoned_empty():
+            return super().forward(*a, **k)
+
+    def forward_only(self, *a, **k):
+        with poisoned_empty():
+            return super().forward_only(*a, **k)
+
+    def backward(self, *a, **k):
+        with poisoned_empty():
+            return super().backward(*a, **k)
 
     def __init__(self, plan, state_meta=None, against_end=True):
         self.plan = plan
