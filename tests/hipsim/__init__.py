@@ -183,12 +183,40 @@ class SimPlan(CompiledPlan):
     def _capturing(self):
         return False
 
+    _WRITTEN = ('out', 'stT', 'sck', 'aux', 'din', 'dst', 'dck', 'daux')      # tensors a kernel stores or accumulates into
+
+    def _tune(self, name, tensors, accumulators=()):
+        self._acc = [(a, a.clone()) for a in accumulators]
+        self._first = None
+        try:
+            super()._tune(name, tensors, accumulators)
+        finally:
+            self._acc, self._first = [], None
+
     def _timed_launch(self, kname, tensors):
         """A launch of the selected candidate; the "time" makes the last candidate the winner of `_tune`, so
-        that the launch after the timing rounds runs a build other than the first."""
+        that the launch after the timing rounds runs a build other than the first.  Every candidate starts from the
+        same accumulator contents and must leave what the first candidate left, up to the order of additions (tiles
+        differ in it): a candidate with wrong values is caught even when another one wins."""
+        for a, saved in getattr(self, '_acc', []):
+            a.copy_(saved)
         self._launch(kname, tensors)
         spec = self.kernels[kname][0]
         index = next(i for i, b in enumerate(self.builds[kname]) if b[0] is spec)
+        got = {n: tensors[n] for n in spec.tensors
+               if n.startswith(self._WRITTEN) and not n.startswith(('dstT', 'dout')) and tensors[n].is_floating_point() and tensors[n].numel()}
+        if getattr(self, '_first', None) is None:
+            self._first = (index, {n: t.clone() for n, t in got.items()})
+        else:
+            i0, ref = self._first
+            self.compared = getattr(self, 'compared', 0) + 1
+            for n, t in got.items():
+                a, b = t.double(), ref[n].double()
+                assert bool((th.isnan(a) == th.isnan(b)).all()), f'{kname}: candidates {i0} and {index} leave different parts of {n} unwritten'
+                a, b = th.nan_to_num(a), th.nan_to_num(b)
+                tol = 2e-2 if t.element_size() == 2 else 1e-4
+                err = (a - b).abs().max().item()
+                assert err <= tol * max(b.abs().max().item(), 1e-30), f'{kname}: candidate {index} differs from candidate {i0} in {n}: {err:.3e}'
         return float(len(self.builds[kname]) - index)
 
     def _launch(self, kname, tensors):

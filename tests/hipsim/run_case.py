@@ -94,7 +94,7 @@ def main():
     print(f'{name} {dims} {dt} tile={plan.tile}', flush=True)
     worst = max(recurrence.assert_all_close(got, want, tol, name))
     ran = sorted({f'{k}#{i}' for k, i in sp.launches})
-    print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e} lds={sp.lds_peak} builds run: {" ".join(ran)}')
+    print(f'{name} {dims} {dt} tile={plan.tile} worst={worst:.3e} lds={sp.lds_peak} candidate launches compared with the first: {getattr(sp, "compared", 0)} builds run: {" ".join(ran)}')
 
 
 if __name__ == '__main__':
