@@ -331,3 +331,78 @@ def test_shipped_picks_are_well_formed_and_name_existing_candidates():
             os.environ.pop('FLEX_RNN_CACHE') if old is None else os.environ.__setitem__('FLEX_RNN_CACHE', old)
     if not matched:
         pytest.skip('the shipped choices were timed on other kernel sources; they are ignored until exported again')
+
+
+def test_kept_row_sums_and_deeper_staging_are_candidates_where_they_apply():
+    """`TileConfig.KS` is a timed candidate of large problems only, per kernel (bit 0 forward, bit 1 reverse scan), and the
+    emitter ignores it where a group of lanes is too small to keep a block's steps; a candidate tile with more waves than the
+    plan's own stages as many timesteps as its larger LDS share holds."""
+    import dataclasses
+    import torch as th
+    import flex_rnn_amd
+    from flex_rnn_amd import examples, launch, planner, prebuild
+    from flex_rnn_amd.emit_hip import Emitter
+    plan = prebuild.plan_for('rwkv7')
+    for reverse in (False, True):
+        bit = 2 if reverse else 1
+        variants = launch.row_kernel_variants(plan, reverse)
+        assert any(v.KS & bit for v in variants) and not any(v.KS & (3 ^ bit) for v in variants)
+    assert all(v.KS == 0 for v in launch.row_kernel_variants(prebuild.plan_for('rwkv7', (2, 64, 2, 128, 128)), False))
+    kept = Emitter(dataclasses.replace(plan, tile=dataclasses.replace(plan.tile, KS=3)))
+    assert 'k_y0' in kept.fw().source and 'k_y0' in kept.fw(save=False).source and 'k_da0' in kept.bw1().source
+    assert 'k_y0' not in Emitter(plan).fw().source
+    m1 = prebuild.plan_for('mamba1')                       # groups of 4 lanes, 16 staged steps: four kept steps per lane, not done
+    assert m1.tile.L == 4 and Emitter(dataclasses.replace(m1, tile=dataclasses.replace(m1.tile, KS=3))).fw().source == Emitter(m1).fw().source
+    # a traced RWKV-7 layer stages ten rows per timestep: 8 timesteps at four waves per workgroup, 16 at eight
+    inputs, layer, _ = examples.build('rwkv7', 8, 1024, 4096, 128, 'meta', raw=True)
+    lay = flex_rnn_amd.layer(layer)
+    lay.graph(*[i.to(th.bfloat16) for i in inputs])
+    call, = lay.calls
+    lplan = planner.make_plan(call.fused.step, *call.metas)[0]
+    assert lplan.tile.TS == 8 and lplan.tile.W == 4
+    for v in launch.row_kernel_variants(lplan, False):
+        assert v.TS == (16 if v.W == 8 else 8)
+        planner.check_tile(v, lplan.H, lplan.NP, lplan.part)
+
+
+def test_first_call_timing_skips_spilling_builds_and_reruns_close_contenders(tmp_path, monkeypatch):
+    """`CompiledPlan._tune`: a build that spills more than `MAX_SPILL_BYTES` per lane is never launched (the first-ranked one
+    aside), and candidates within 3 % of the fastest are run again by themselves and ranked by their medians."""
+    from flex_rnn_amd import launch, prebuild
+    from flex_rnn_amd.emit_hip import KernelSpec
+    monkeypatch.setenv('FLEX_RNN_CACHE', str(tmp_path))
+    monkeypatch.delenv('FLEX_RNN_RETUNE', raising=False)
+    plan = prebuild.plan_for('rwkv7', (2, 64, 2, 128, 128))
+
+    class Fake:
+        _tune_rounds = 3
+        _tune = launch.CompiledPlan._tune
+
+        def __init__(self, spills, ms):
+            self.plan, self.ms, self.launched, self.sel = plan, ms, [], None
+            self.builds = {'frnn_bw2': [(KernelSpec('frnn_bw2', f'// build {i} {spills} {ms}', [], 64, ('1', '1', '1'), {}), None,
+                                         {'scratch': s_, 'occupancy': 2, 'vgprs': 128}) for i, s_ in enumerate(spills)]}
+            self._tune_pending, self.build_times, self.build_source = {'frnn_bw2'}, {}, {}
+
+        def _capturing(self):
+            return False
+
+        def _device_name(self):
+            return 'test-device'
+
+        def _select(self, name, i):
+            self.sel = i
+
+        def _timed_launch(self, name, tensors):
+            self.launched.append(self.sel)
+            v = self.ms[self.sel]
+            return v(len(self.launched)) if callable(v) else v
+
+    f = Fake([0, 200, 20, 65], [3.0, 0.5, 2.0, 0.1])
+    f._tune('frnn_bw2', {})
+    assert set(f.launched) == {0, 2} and f.sel == 2 and f.build_times['frnn_bw2'][1] == float('inf')
+    # two contenders within 3 %: the one with a single lucky run loses on the median
+    lucky = iter([0.95] + [1.02] * 100)
+    f = Fake([0, 0, 0], [1.0, lambda n: next(lucky), 1.5])
+    f._tune('frnn_bw2', {})
+    assert f.sel == 0 and f.launched.count(2) == 3 and f.launched.count(0) == 3 + 6 and f.launched.count(1) == 3 + 6
